@@ -9,7 +9,9 @@ Groups: cache slabs whose mixers have the same need (heads, head size, window)
 form a group with a page pool and block tables of its own.  A request's block
 table in a group lists its pages in token order; all slabs of the group use the
 same page ids.  A group with a window gives pages back as soon as every token in
-them lies behind the window of the next token; their table entries become -1.
+them lies behind the window of the next token; their table entries become -1.  A group
+whose need names `keep_first` tokens never gives back the pages that hold a request's first
+tokens of that count: they stay visible beside the window.
 
 Protocol for one step: `reserve(req, n)` takes the pages that the next n tokens
 need in every group (all or nothing; `reserve_step` does it for all requests of a
@@ -52,11 +54,11 @@ def _library():
         from ..csrc import build
 
         lib = ctypes.CDLL(build.ensure_host_built())
-        if lib.egh_abi_version() != 3:
+        if lib.egh_abi_version() != 4:
             raise RuntimeError("the host library has an unexpected ABI version")
         vp, i = ctypes.c_void_p, ctypes.c_int
         sigs = {
-            "egh_create": ([i, vp, vp, i, i], vp), "egh_destroy": ([vp], None), "egh_admit": ([vp], i),
+            "egh_create": ([i, vp, vp, i, i], vp), "egh_destroy": ([vp], None), "egh_set_keep_first": ([vp, i, i], i), "egh_admit": ([vp], i),
             "egh_release": ([vp, i], i), "egh_slot": ([vp, i], i), "egh_num_tokens": ([vp, i], i),
             "egh_version": ([vp, i], i), "egh_table_len": ([vp, i, i], i), "egh_table": ([vp, i, i, vp, i], i),
             "egh_pages_needed": ([vp, i, i, vp], i), "egh_free_pages": ([vp, i], i), "egh_used_pages": ([vp, i], i),
@@ -152,6 +154,10 @@ class CacheManager:
         self._core = self._lib.egh_create(len(self.groups), _ints(windows), _ints(counts), self.page_size, int(max_requests))
         if not self._core:
             raise ValueError("the cache manager could not be created from these sizes")
+        for g, need in enumerate(self.groups):
+            keep = int(getattr(need, "keep_first", 0) or 0)
+            if keep and self._lib.egh_set_keep_first(self._core, g, keep) != 0:
+                raise ValueError(f"cache group {g}: keep_first {keep} was refused")
         self.pools = [PoolView(n) for n in counts]
         self.slots = SlotView(int(max_requests))
         self.requests: dict[object, RequestCache] = {}

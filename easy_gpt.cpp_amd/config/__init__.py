@@ -1,4 +1,5 @@
 from .base import ConfigError, KeyReader, read_json
+from .pekasun import PekasunConfig
 from .qwen2 import Qwen2Config
 from .registry import (
     Architecture,
@@ -14,6 +15,7 @@ __all__ = [
     "Architecture",
     "ConfigError",
     "KeyReader",
+    "PekasunConfig",
     "Qwen2Config",
     "UnknownArchitectureError",
     "load_model_config",

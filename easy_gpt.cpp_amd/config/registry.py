@@ -66,10 +66,13 @@ def _ensure_builtin() -> None:
 
 
 def resolve_architecture(config: Mapping[str, Any]) -> Architecture:
-    """Architecture named by a config.json mapping: ``architectures[0]`` first, then ``model_type``."""
+    """Architecture named by a config.json mapping: ``architectures[0]`` (or the single name in ``architecture``)
+    first, then ``model_type``."""
     _ensure_builtin()
     archs = config.get("architectures")
     name = archs[0] if isinstance(archs, list) and archs and isinstance(archs[0], str) else ""
+    if not name and isinstance(config.get("architecture"), str):
+        name = config["architecture"]
     model_type = config.get("model_type") if isinstance(config.get("model_type"), str) else ""
     if name in _BY_NAME:
         return _BY_NAME[name]

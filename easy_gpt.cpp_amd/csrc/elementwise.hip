@@ -5,31 +5,6 @@
 
 namespace egpt {
 
-// The output of a product arrives either as one tensor of the activation type, or as float32 partial
-// sums [n_splits][rows][cols] of a split-k product, which are added here in split order.
-template <typename T>
-struct ProductView {
-    const T* whole;          // used when n_splits == 0
-    const float* partial;    // used when n_splits > 0
-    int n_splits;
-    size_t split_stride;     // rows * cols
-    __device__ __forceinline__ bool present() const { return whole != nullptr || partial != nullptr; }
-    __device__ __forceinline__ float at(size_t idx) const {
-        if (n_splits == 0) return to_float(whole[idx]);
-        // up to sixteen loads in flight at a time (a chain of dependent kernels pays for round trips, not
-        // bytes); the order of the additions is fixed
-        float v = 0.f;
-        for (int s0 = 0; s0 < n_splits; s0 += 16) {
-            float t[16];
-#pragma unroll
-            for (int i = 0; i < 16; ++i) t[i] = s0 + i < n_splits ? partial[(s0 + i) * split_stride + idx] : 0.f;
-#pragma unroll
-            for (int i = 0; i < 16; ++i) v += t[i];
-        }
-        return v;
-    }
-};
-
 // ----------------------------------------------------------------------------- embedding
 // x[t, :] = E[id_t, :]   (/root/reference/src/models/embedding.cpp:54-76); output: the residual stream, float32 or
 // fixed point.
@@ -624,4 +599,4 @@ extern "C" const char* egpt_error_string(int code) {
     }
 }
 
-extern "C" int egpt_abi_version(void) { return 16; }
+extern "C" int egpt_abi_version(void) { return 17; }

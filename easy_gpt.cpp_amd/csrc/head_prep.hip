@@ -1,0 +1,277 @@
+// What stands between a mixer's input product and its attention, head by head, for mixers that norm or rotate
+// single heads: an embedding gather with its norm, per-head RMS norms of queries, keys and values with the store
+// into cache pages, the preparation of latent attention (latent norm, interleaved rotation of the rotated parts,
+// store of latent and rotated key), and a sigmoid gate.  Statistics, angles and the rotation are float32; values
+// are rounded once, when they are written in the activation type.
+//
+// A product arrives as one tensor of the activation type or as float32 partial sums (ProductView in common.h).
+// Keys lie in pages [page][kv head][offset][key size], values in pages [page][kv head][value size][offset].
+#include "api.h"
+#include "common.h"
+
+namespace egpt {
+
+constexpr int kMaxHeadWidth = 1024;                   // the widest head (or latent) these kernels take
+constexpr int kOwn = kMaxHeadWidth / kWave;           // values of it that a lane keeps
+
+// x[t, :] = E[id_t, :] / sqrt(mean(E[id_t, :]^2) + eps) * w, written as the float32 residual stream.
+template <typename T>
+__global__ __launch_bounds__(256) void embed_rmsnorm_kernel(const int32_t* __restrict__ ids, const T* __restrict__ table,
+                                                            const T* __restrict__ weight, float eps,
+                                                            float* __restrict__ out, int hidden, int vocab) {
+    __shared__ float scratch[16];
+    const int t = blockIdx.x;
+    int id = ids[t];
+    id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);      // ids are range-checked on the host; never read outside
+    const T* row = table + static_cast<size_t>(id) * hidden;
+    float ss = 0.f;
+    for (int j = threadIdx.x; j < hidden; j += blockDim.x) {
+        const float v = to_float(row[j]);
+        ss = fmaf(v, v, ss);
+    }
+    ss = block_sum(ss, scratch);
+    const float inv = inv_rms(ss, 1.0f / static_cast<float>(hidden), eps);
+    float* o = out + static_cast<size_t>(t) * hidden;
+    for (int j = threadIdx.x; j < hidden; j += blockDim.x) o[j] = to_float(row[j]) * inv * to_float(weight[j]);
+}
+
+// One wavefront per (token, head) of a product row [nq heads of dk | nkv heads of dk | nkv heads of dv]: a query or
+// key head is divided by its root mean square and multiplied by the weight that all heads share (a null weight:
+// the head passes as it is), a value head is divided by its root mean square if norm_values is set.  Queries go
+// to q_out [T][nq * dk]; keys and values to the pages at slots[t] (slots null: nothing is stored).
+template <typename T>
+__global__ __launch_bounds__(kWave) void head_norm_store_kernel(
+    ProductView<T> proj, T* __restrict__ q_out, const T* __restrict__ q_weight, const T* __restrict__ k_weight, float eps,
+    int norm_values, const int32_t* __restrict__ slots, T* __restrict__ k_cache, T* __restrict__ v_cache, int nq, int nkv,
+    int dk, int dv, int page_size) {
+    const int t = blockIdx.x, hh = blockIdx.y, lane = threadIdx.x;
+    const int row_width = (nq + nkv) * dk + nkv * dv;
+    const int kind = hh < nq ? 0 : (hh < nq + nkv ? 1 : 2);
+    const int head = kind == 0 ? hh : (kind == 1 ? hh - nq : hh - nq - nkv);
+    const int width = kind == 2 ? dv : dk;
+    const int in_off = kind == 0 ? head * dk : (kind == 1 ? nq * dk + head * dk : (nq + nkv) * dk + head * dv);
+    if (kind != 0 && slots == nullptr) return;
+    const T* weight = kind == 0 ? q_weight : (kind == 1 ? k_weight : nullptr);
+    const bool normed = kind == 2 ? norm_values != 0 : weight != nullptr;
+    const size_t base = static_cast<size_t>(t) * row_width + in_off;
+    float v[kOwn];
+    float ss = 0.f;
+#pragma unroll
+    for (int r = 0; r < kOwn; ++r) {
+        const int d = lane + r * kWave;
+        v[r] = d < width ? proj.at(base + d) : 0.f;
+        ss = fmaf(v[r], v[r], ss);
+    }
+    float inv = 1.0f;
+    if (normed) inv = inv_rms(wave_sum(ss), 1.0f / static_cast<float>(width), eps);
+    long page = 0;
+    int off = 0;
+    if (kind != 0) {
+        page = slots[t] / page_size;
+        off = slots[t] % page_size;
+    }
+#pragma unroll
+    for (int r = 0; r < kOwn; ++r) {
+        const int d = lane + r * kWave;
+        if (d >= width) continue;
+        float y = v[r] * inv;
+        if (weight != nullptr) y *= to_float(weight[d]);
+        if (kind == 0)
+            q_out[static_cast<size_t>(t) * nq * dk + head * dk + d] = from_float<T>(y);
+        else if (kind == 1)
+            k_cache[((page * nkv + head) * page_size + off) * dk + d] = from_float<T>(y);
+        else
+            v_cache[((page * nkv + head) * dv + d) * page_size + off] = from_float<T>(y);
+    }
+}
+
+// One wavefront per (token, query head) and one more per token for the latent, of a product row
+// [nq heads of (dim unrotated | rot rotated) | rank latent | rot shared rotated key | anything else].
+// A query head's unrotated part goes to q_plain [T][nq][dim], its rotated part, rotated, to q_full [T][nq][rank + rot]
+// behind the first rank places (which the caller fills with the unrotated part carried into the latent space).
+// The latent is divided by its root mean square and multiplied by c_weight; with the rotated shared key behind it
+// it is the token's key [rank + rot] in the pages, and alone, transposed, its value [rank].
+// Rotation: the pair (2i, 2i + 1) of the rotated part, i < rot_dims / 2, by the angle whose (cos, sin) stand in
+// cos_sin [T][rot_dims / 2][2]; both are multiplied by mag; places from rot_dims on pass unchanged.
+template <typename T>
+__global__ __launch_bounds__(kWave) void latent_prep_kernel(
+    ProductView<T> proj, int row_width, T* __restrict__ q_plain, T* __restrict__ q_full, const T* __restrict__ c_weight,
+    float eps, const float* __restrict__ cos_sin, float mag, int rot_dims, const int32_t* __restrict__ slots,
+    T* __restrict__ k_cache, T* __restrict__ v_cache, int nq, int dim, int rot, int rank, int page_size) {
+    const int t = blockIdx.x, hh = blockIdx.y, lane = threadIdx.x;
+    const size_t row = static_cast<size_t>(t) * row_width;
+    const float* cs = cos_sin + static_cast<size_t>(t) * rot_dims;      // (rot_dims / 2) pairs of (cos, sin)
+    const int dk = rank + rot;
+    if (hh < nq) {
+        const size_t base = row + static_cast<size_t>(hh) * (dim + rot);
+        for (int d = lane; d < dim; d += kWave)
+            q_plain[(static_cast<size_t>(t) * nq + hh) * dim + d] = from_float<T>(proj.at(base + d));
+        T* dst = q_full + (static_cast<size_t>(t) * nq + hh) * dk + rank;
+        for (int i = lane; i < rot / 2; i += kWave) {
+            const float u = proj.at(base + dim + 2 * i), w = proj.at(base + dim + 2 * i + 1);
+            float ru = u, rw = w;
+            if (2 * i + 1 < rot_dims) rotate_pair(u, w, cs[2 * i] * mag, cs[2 * i + 1] * mag, ru, rw);
+            dst[2 * i] = from_float<T>(ru);
+            dst[2 * i + 1] = from_float<T>(rw);
+        }
+        if ((rot & 1) && lane == 0) dst[rot - 1] = from_float<T>(proj.at(base + dim + rot - 1));
+        return;
+    }
+    if (slots == nullptr) return;
+    const size_t base = row + static_cast<size_t>(nq) * (dim + rot);
+    float v[kOwn];
+    float ss = 0.f;
+#pragma unroll
+    for (int r = 0; r < kOwn; ++r) {
+        const int d = lane + r * kWave;
+        v[r] = d < rank ? proj.at(base + d) : 0.f;
+        ss = fmaf(v[r], v[r], ss);
+    }
+    const float inv = inv_rms(wave_sum(ss), 1.0f / static_cast<float>(rank), eps);
+    const long page = slots[t] / page_size;
+    const int off = slots[t] % page_size;
+    T* kdst = k_cache + (page * page_size + off) * dk;
+    T* vdst = v_cache + page * rank * page_size + off;
+#pragma unroll
+    for (int r = 0; r < kOwn; ++r) {
+        const int d = lane + r * kWave;
+        if (d >= rank) continue;
+        const T y = from_float<T>(v[r] * inv * to_float(c_weight[d]));
+        kdst[d] = y;
+        vdst[static_cast<long>(d) * page_size] = y;
+    }
+    for (int i = lane; i < rot / 2; i += kWave) {
+        const float u = proj.at(base + rank + 2 * i), w = proj.at(base + rank + 2 * i + 1);
+        float ru = u, rw = w;
+        if (2 * i + 1 < rot_dims) rotate_pair(u, w, cs[2 * i] * mag, cs[2 * i + 1] * mag, ru, rw);
+        kdst[rank + 2 * i] = from_float<T>(ru);
+        kdst[rank + 2 * i + 1] = from_float<T>(rw);
+    }
+    if ((rot & 1) && lane == 0) kdst[rank + rot - 1] = from_float<T>(proj.at(base + rank + rot - 1));
+}
+
+// out[t][n] = x[t][n] * sigmoid(g[t][gate_off + n]); x lies [T][N], or with heads > 0 head by head [heads][T][N / heads]
+// (what a product batched over heads leaves).  g: columns of a product row of width gate_width.
+template <typename T>
+__global__ __launch_bounds__(256) void sigmoid_gate_kernel(const T* __restrict__ x, int heads, ProductView<T> g,
+                                                           int gate_width, int gate_off, T* __restrict__ out,
+                                                           int n_tokens, int n) {
+    const size_t idx = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (idx >= static_cast<size_t>(n_tokens) * n) return;
+    const int t = static_cast<int>(idx / n), c = static_cast<int>(idx % n);
+    size_t src = idx;
+    if (heads > 0) {
+        const int per = n / heads;
+        src = (static_cast<size_t>(c / per) * n_tokens + t) * per + c % per;
+    }
+    const float gate = g.at(static_cast<size_t>(t) * gate_width + gate_off + c);
+    out[idx] = from_float<T>(to_float(x[src]) * (1.0f / (1.0f + expf(-gate))));
+}
+
+template <typename T>
+static ProductView<T> view_of(const void* p, int n_splits, size_t split_stride) {
+    ProductView<T> v;
+    v.whole = n_splits == 0 ? static_cast<const T*>(p) : nullptr;
+    v.partial = n_splits > 0 ? static_cast<const float*>(p) : nullptr;
+    v.n_splits = n_splits;
+    v.split_stride = split_stride;
+    return v;
+}
+
+}  // namespace egpt
+
+using namespace egpt;
+
+extern "C" int egpt_embed_rmsnorm(const int32_t* ids, const void* table, const void* weight, float eps, float* out,
+                                  int n_tokens, int hidden, int vocab, int dtype, void* stream) {
+    if (!ids || !table || !weight || !out || n_tokens < 0 || hidden <= 0 || vocab <= 0 || (dtype != 0 && dtype != 1))
+        return EGPT_BAD_ARGUMENT;
+    if (n_tokens == 0) return EGPT_OK;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (dtype == 0)
+        embed_rmsnorm_kernel<<<n_tokens, 256, 0, s>>>(ids, static_cast<const float*>(table),
+                                                      static_cast<const float*>(weight), eps, out, hidden, vocab);
+    else
+        embed_rmsnorm_kernel<<<n_tokens, 256, 0, s>>>(ids, static_cast<const bf16_t*>(table),
+                                                      static_cast<const bf16_t*>(weight), eps, out, hidden, vocab);
+    EGPT_CHECK_LAUNCH();
+    return EGPT_OK;
+}
+
+extern "C" int egpt_head_norm_store(const void* proj, int n_splits, void* q_out, const void* q_weight,
+                                    const void* k_weight, float eps, int norm_values, const int32_t* slots,
+                                    void* k_cache, void* v_cache, int n_tokens, int nq, int nkv, int dk, int dv,
+                                    int page_size, int dtype, void* stream) {
+    if (!proj || !q_out || n_splits < 0 || n_tokens < 0 || nq <= 0 || nkv <= 0 || dk <= 0 || dv <= 0 || page_size <= 0 ||
+        (dtype != 0 && dtype != 1))
+        return EGPT_BAD_ARGUMENT;
+    if (slots && (!k_cache || !v_cache)) return EGPT_BAD_ARGUMENT;
+    if (dk > kMaxHeadWidth || dv > kMaxHeadWidth || nq + 2 * nkv > 65535) return EGPT_UNSUPPORTED_SIZE;
+    if (n_tokens == 0) return EGPT_OK;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const size_t stride = static_cast<size_t>(n_tokens) * ((nq + nkv) * dk + nkv * dv);
+    dim3 grid(n_tokens, nq + 2 * nkv);
+    if (dtype == 0)
+        head_norm_store_kernel<float><<<grid, kWave, 0, s>>>(
+            view_of<float>(proj, n_splits, stride), static_cast<float*>(q_out), static_cast<const float*>(q_weight),
+            static_cast<const float*>(k_weight), eps, norm_values, slots, static_cast<float*>(k_cache),
+            static_cast<float*>(v_cache), nq, nkv, dk, dv, page_size);
+    else
+        head_norm_store_kernel<bf16_t><<<grid, kWave, 0, s>>>(
+            view_of<bf16_t>(proj, n_splits, stride), static_cast<bf16_t*>(q_out), static_cast<const bf16_t*>(q_weight),
+            static_cast<const bf16_t*>(k_weight), eps, norm_values, slots, static_cast<bf16_t*>(k_cache),
+            static_cast<bf16_t*>(v_cache), nq, nkv, dk, dv, page_size);
+    EGPT_CHECK_LAUNCH();
+    return EGPT_OK;
+}
+
+extern "C" int egpt_latent_prep(const void* proj, int n_splits, int row_width, void* q_plain, void* q_full,
+                                const void* c_weight, float eps, const float* cos_sin, float mag, int rot_dims,
+                                const int32_t* slots, void* k_cache, void* v_cache, int n_tokens, int nq, int dim,
+                                int rot, int rank, int page_size, int dtype, void* stream) {
+    if (!proj || !q_plain || !q_full || !c_weight || n_splits < 0 || n_tokens < 0 || nq <= 0 || dim <= 0 || rot < 0 ||
+        rank <= 0 || page_size <= 0 || rot_dims < 0 || rot_dims > rot || rot_dims % 2 || (dtype != 0 && dtype != 1))
+        return EGPT_BAD_ARGUMENT;
+    if (rot_dims > 0 && !cos_sin) return EGPT_BAD_ARGUMENT;
+    if (slots && (!k_cache || !v_cache)) return EGPT_BAD_ARGUMENT;
+    if (row_width < nq * (dim + rot) + rank + rot) return EGPT_BAD_ARGUMENT;
+    if (rank > kMaxHeadWidth || nq + 1 > 65535) return EGPT_UNSUPPORTED_SIZE;
+    if (n_tokens == 0) return EGPT_OK;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const size_t stride = static_cast<size_t>(n_tokens) * row_width;
+    dim3 grid(n_tokens, nq + 1);
+    if (dtype == 0)
+        latent_prep_kernel<float><<<grid, kWave, 0, s>>>(
+            view_of<float>(proj, n_splits, stride), row_width, static_cast<float*>(q_plain), static_cast<float*>(q_full),
+            static_cast<const float*>(c_weight), eps, cos_sin, mag, rot_dims, slots, static_cast<float*>(k_cache),
+            static_cast<float*>(v_cache), nq, dim, rot, rank, page_size);
+    else
+        latent_prep_kernel<bf16_t><<<grid, kWave, 0, s>>>(
+            view_of<bf16_t>(proj, n_splits, stride), row_width, static_cast<bf16_t*>(q_plain),
+            static_cast<bf16_t*>(q_full), static_cast<const bf16_t*>(c_weight), eps, cos_sin, mag, rot_dims, slots,
+            static_cast<bf16_t*>(k_cache), static_cast<bf16_t*>(v_cache), nq, dim, rot, rank, page_size);
+    EGPT_CHECK_LAUNCH();
+    return EGPT_OK;
+}
+
+extern "C" int egpt_sigmoid_gate(const void* x, int heads, const void* gate, int gate_splits, int gate_width,
+                                 int gate_off, void* out, int n_tokens, int n, int dtype, void* stream) {
+    if (!x || !gate || !out || n_tokens < 0 || n <= 0 || heads < 0 || (heads > 0 && n % heads) || gate_splits < 0 ||
+        gate_off < 0 || gate_off + n > gate_width || (dtype != 0 && dtype != 1))
+        return EGPT_BAD_ARGUMENT;
+    if (n_tokens == 0) return EGPT_OK;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const size_t total = static_cast<size_t>(n_tokens) * n;
+    const size_t stride = static_cast<size_t>(n_tokens) * gate_width;
+    const unsigned blocks = static_cast<unsigned>((total + 255) / 256);
+    if (dtype == 0)
+        sigmoid_gate_kernel<float><<<blocks, 256, 0, s>>>(static_cast<const float*>(x), heads,
+                                                          view_of<float>(gate, gate_splits, stride), gate_width, gate_off,
+                                                          static_cast<float*>(out), n_tokens, n);
+    else
+        sigmoid_gate_kernel<bf16_t><<<blocks, 256, 0, s>>>(static_cast<const bf16_t*>(x), heads,
+                                                           view_of<bf16_t>(gate, gate_splits, stride), gate_width,
+                                                           gate_off, static_cast<bf16_t*>(out), n_tokens, n);
+    EGPT_CHECK_LAUNCH();
+    return EGPT_OK;
+}

@@ -50,6 +50,7 @@ struct Request {
 struct EghCore {
     int page_size = 1;
     std::vector<int> windows;
+    std::vector<int> keep_first;      // per group: tokens at the start of a request that a window never lets go
     std::vector<Pool> pools;
     std::vector<int32_t> free_slots;
     std::vector<uint8_t> slot_held;
@@ -66,7 +67,7 @@ struct EghCore {
 
 extern "C" {
 
-int egh_abi_version(void) { return 3; }
+int egh_abi_version(void) { return 4; }
 
 EghCore* egh_create(int n_groups, const int32_t* windows, const int32_t* num_pages, int page_size, int max_requests) {
     if (n_groups < 0 || page_size < 1 || max_requests < 0 || (n_groups > 0 && (!windows || !num_pages))) return nullptr;
@@ -75,6 +76,7 @@ EghCore* egh_create(int n_groups, const int32_t* windows, const int32_t* num_pag
     EghCore* c = new EghCore();
     c->page_size = page_size;
     c->windows.assign(windows, windows + n_groups);
+    c->keep_first.assign(n_groups, 0);
     c->pools.resize(n_groups);
     for (int g = 0; g < n_groups; ++g) c->pools[g].init(num_pages[g]);
     c->free_slots.resize(max_requests);
@@ -84,6 +86,14 @@ EghCore* egh_create(int n_groups, const int32_t* windows, const int32_t* num_pag
 }
 
 void egh_destroy(EghCore* c) { delete c; }
+
+int egh_set_keep_first(EghCore* c, int g, int n) {
+    if (!c || g < 0 || g >= c->n_groups() || n < 0) return EGH_BAD_ARGUMENT;
+    for (const Request& r : c->requests)
+        if (r.live) return EGH_BAD_ARGUMENT;
+    c->keep_first[g] = n;
+    return EGH_OK;
+}
 
 int egh_admit(EghCore* c) {
     if (!c) return EGH_BAD_ARGUMENT;
@@ -232,8 +242,9 @@ int egh_commit(EghCore* c, int n, const int32_t* handles, const int32_t* counts)
             // the next token (position num_tokens) reads keys j > num_tokens - window
             const int first_needed = r->num_tokens - window + 1;
             const int dead = std::max(0, first_needed) / c->page_size;        // pages wholly below first_needed
+            const int kept = c->pages_for(c->keep_first[g]);                  // pages that hold a kept first token
             bool changed = false;
-            for (int j = 0; j < dead; ++j) {
+            for (int j = kept; j < dead; ++j) {
                 int32_t& p = r->tables[g][j];
                 if (p >= 0) {
                     if (!c->pools[g].give_back(p)) return EGH_INVARIANT;

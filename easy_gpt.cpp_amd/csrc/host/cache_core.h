@@ -21,6 +21,9 @@ int egh_abi_version(void);
 // windows[g] == 0: the group keeps every key.  num_pages[g] pages of page_size tokens; max_requests slots.
 EghCore* egh_create(int n_groups, const int32_t* windows, const int32_t* num_pages, int page_size, int max_requests);
 void egh_destroy(EghCore* c);
+// The first n tokens of every request stay readable in group g however far its window has moved on: the pages that
+// hold them are never given back before the request ends.  Before any request is admitted.
+int egh_set_keep_first(EghCore* c, int g, int n);
 
 int egh_admit(EghCore* c);                                  // a handle >= 0, or EGH_NO_SLOT
 int egh_release(EghCore* c, int h);                         // pages and slot go back

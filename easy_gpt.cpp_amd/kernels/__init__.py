@@ -32,6 +32,27 @@ Methods of a backend (T tokens, B requests, R rows, act = bfloat16 or float32):
   argmax(logits f32[R,V], out i32[R])            lowest index among equal maxima
   sample(logits f32[R,V], temperature f32[R], top_k i32[R], top_p f32[R], uniform f32[R], out i32[R])
 
+  embed_rmsnorm(token_ids i32[T], table act[V,H], weight act[H], eps, out f32[T,H])
+        out = table[id] / sqrt(mean(table[id]^2) + eps) * weight: an embedding with its norm, as the residual stream
+  head_norm_store(proj act[T,W]|f32[S,T,W], q_out act[T,nq*dk], q_weight act[dk]|None, k_weight act[dk]|None, eps,
+                  norm_values, slots i32[T]|None, k_cache, v_cache, nq, nkv, dk, dv, page_size)
+        proj rows are [nq heads of dk | nkv heads of dk | nkv heads of dv]; query and key heads are divided by their
+        root mean square and multiplied by the weight (None: they pass), value heads are divided by theirs if
+        norm_values; queries to q_out, keys [P,nkv,page_size,dk] and values [P,nkv,dv,page_size] to `slots`
+  latent_prep(proj, q_plain act[T,nq,dim], q_full act[T,nq,rank+rot], c_weight act[rank], eps, cos_sin f32[T,rd/2,2]|None,
+              magnitude, rotary_dim, slots, k_cache, v_cache, nq, dim, rot, rank, page_size)
+        proj rows are [nq heads of (dim | rot) | rank | rot | ...]; the heads' unrotated parts to q_plain, their rotated
+        parts (pairs (2i, 2i+1) of the first rotary_dim places turned by the table's angles, cos and sin times
+        magnitude) to q_full[..., rank:]; the latent, RMS-normed with c_weight, with the rotated shared key behind it
+        as key [P,1,page_size,rank+rot], the latent alone as value [P,1,rank,page_size], at `slots`
+  heads_product(x act[heads,T,K] (any strides), w act[heads,K,N]) -> act[heads,T,N]    one product per head
+  sigmoid_gate(x act[T,N] | act[heads,T,N/heads], heads, gate act[T,W]|f32[S,T,W], gate_offset, out act[T,N])
+        out = x * sigmoid(gate[:, gate_offset : gate_offset + N])
+  window_attention(q act[T,nq*dk], out act[T,nq*dv], k_cache, v_cache, block_table, q_start, q_len, kv_len, nq, nkv,
+                   dk, dv, page_size, scale, window, keep_first, sink f32[nq]|None, max_q_len, max_kv_len)
+        as paged_attention with key size dk and value size dv; key j <= p is read if window == 0, p - j < window or
+        j < keep_first; with a sink the softmax's denominator also holds exp(sink[head])
+
 Beside these, a backend has fused variants that fold neighbouring operations into one kernel.  They are part of
 the contract too (`KernelBackend` below): each returns None (False for the decode attention) where it does not
 cover a case, and the caller then takes the unfused way.
@@ -50,6 +71,7 @@ class KernelBackend:
     name = "abstract"
     max_head_dim = 256      # the widest attention head the kernels take: a part refuses more when it is built
     fused_rows = 0          # products whose x operand is computed while it is staged take at most this many rows
+    max_window_attention_dim = 1024     # the widest key or value that window_attention takes
 
     def pinned_stream(self):
         """Context manager within which every launch goes to the stream that is current on entry."""
@@ -79,6 +101,13 @@ class KernelBackend:
         import torch
 
         return (h.double() * (1.0 / 4294967296.0)).float() if h.dtype == torch.int64 else h
+
+    def heads_product(self, x, w):
+        """x[h] w[h] for every head h: x act [heads, T, K] (any strides), w act [heads, K, N] -> act [heads, T, N].
+        The library's batched product (float32 operands are multiplied in float32)."""
+        import torch
+
+        return torch.bmm(x, w)
 
     def product(self, x, w, unrounded=False, residual=None):
         """x w^T as act [m, n], or as float32 partial sums [splits, m, n] for a consumer that adds them up; or, given

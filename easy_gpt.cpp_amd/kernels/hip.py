@@ -28,7 +28,7 @@ def _load_library() -> ctypes.CDLL:
         lib = ctypes.CDLL(path)
     except (build.BuildError, OSError) as e:
         raise KernelsUnavailable(f"the HIP kernel library could not be built or loaded: {e}") from e
-    if lib.egpt_abi_version() != 16:
+    if lib.egpt_abi_version() != 17:
         raise KernelsUnavailable(f"{path} has an unexpected ABI version")
     return lib
 
@@ -101,6 +101,11 @@ class HipKernels(KernelBackend):
             "egpt_sample": [vp, vp, vp, vp, vp, vp, vp, i, i, vp],
             "egpt_sample_wide": [vp, vp, vp, vp, vp, vp, vp, i, i, vp],
             "egpt_gemm_gate_up_swiglu": [vp, vp, vp, i, i, i, i, vp],
+            "egpt_embed_rmsnorm": [vp, vp, vp, f, vp, i, i, i, i, vp],
+            "egpt_head_norm_store": [vp, i, vp, vp, vp, f, i, vp, vp, vp, i, i, i, i, i, i, i, vp],
+            "egpt_latent_prep": [vp, i, i, vp, vp, vp, f, vp, f, i, vp, vp, vp, i, i, i, i, i, i, i, vp],
+            "egpt_sigmoid_gate": [vp, i, vp, i, i, i, vp, i, i, i, vp],
+            "egpt_window_attention": [vp, vp, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, i, f, i, i, vp, i, vp],
         }
         lib.egpt_sample_workspace.restype = ctypes.c_size_t
         lib.egpt_sample_workspace.argtypes = [i, i]
@@ -844,6 +849,105 @@ class HipKernels(KernelBackend):
                   table_width, q_start.data_ptr(), kv_len.data_ptr(), b, nq, nkv, hd, page_size, float(scale),
                   int(window), n_splits, n_waves, 1 if combine else 0, lean, self._stream())
         return (part_o, part_ml) if (n_splits > 1 and not combine) else None
+
+    # ------------------------------------------------------------------ mixers that treat single heads
+    def embed_rmsnorm(self, token_ids, table, weight, eps, out):
+        dt = self._act(table, "table")
+        v, h = table.shape
+        t = token_ids.shape[0]
+        self._need(token_ids, "token_ids", _I32, (t,))
+        self._need(table, "table")
+        self._need(weight, "weight", table.dtype, (h,))
+        self._need(out, "out", _F32, (t, h))
+        self._run("egpt_embed_rmsnorm", token_ids.data_ptr(), table.data_ptr(), weight.data_ptr(), float(eps),
+                  out.data_ptr(), t, h, v, dt, self._stream())
+
+    def _key_value_pages(self, k_cache, v_cache, dtype, nkv: int, page_size: int, dk: int, dv: int) -> None:
+        self._need(k_cache, "k_cache", dtype)
+        self._need(v_cache, "v_cache", dtype)
+        if k_cache.dim() != 4 or tuple(k_cache.shape[1:]) != (nkv, page_size, dk):
+            raise ValueError(f"k_cache must be [pages, {nkv}, {page_size}, {dk}], got {tuple(k_cache.shape)}")
+        if v_cache.dim() != 4 or tuple(v_cache.shape[1:]) != (nkv, dv, page_size):
+            raise ValueError(f"v_cache must be [pages, {nkv}, {dv}, {page_size}], got {tuple(v_cache.shape)}")
+        if v_cache.shape[0] != k_cache.shape[0]:
+            raise ValueError("k_cache and v_cache must have the same number of pages")
+
+    def head_norm_store(self, proj, q_out, q_weight, k_weight, eps, norm_values, slots, k_cache, v_cache, nq, nkv, dk, dv,
+                        page_size):
+        t = proj.shape[-2]
+        dt = self._act(q_out, "q_out")
+        splits = self._product(proj, "proj", q_out.dtype, t, (nq + nkv) * dk + nkv * dv)
+        self._need(q_out, "q_out", None, (t, nq * dk))
+        for name, w in (("q_weight", q_weight), ("k_weight", k_weight)):
+            if w is not None:
+                self._need(w, name, q_out.dtype, (dk,))
+        if slots is not None:
+            self._need(slots, "slots", _I32, (t,))
+            self._key_value_pages(k_cache, v_cache, q_out.dtype, nkv, page_size, dk, dv)
+        self._run("egpt_head_norm_store", proj.data_ptr(), splits, q_out.data_ptr(), self._ptr(q_weight),
+                  self._ptr(k_weight), float(eps), 1 if norm_values else 0, self._ptr(slots),
+                  self._ptr(k_cache) if slots is not None else None, self._ptr(v_cache) if slots is not None else None,
+                  t, nq, nkv, dk, dv, page_size, dt, self._stream())
+
+    def latent_prep(self, proj, q_plain, q_full, c_weight, eps, cos_sin, magnitude, rotary_dim, slots, k_cache, v_cache,
+                    nq, dim, rot, rank, page_size):
+        t, width = proj.shape[-2], proj.shape[-1]
+        dt = self._act(q_full, "q_full")
+        if width < nq * (dim + rot) + rank + rot:
+            raise ValueError(f"proj rows of {width} values cannot hold {nq} heads of {dim} + {rot}, a latent of {rank} and "
+                             f"a rotated key of {rot}")
+        splits = self._product(proj, "proj", q_full.dtype, t, width)
+        self._need(q_plain, "q_plain", q_full.dtype, (t, nq, dim))
+        self._need(q_full, "q_full", None, (t, nq, rank + rot))
+        self._need(c_weight, "c_weight", q_full.dtype, (rank,))
+        if rotary_dim:
+            if rotary_dim % 2 or rotary_dim > rot:
+                raise ValueError(f"rotary_dim {rotary_dim} must be even and <= the rotated size {rot}")
+            self._need(cos_sin, "cos_sin", _F32, (t, rotary_dim // 2, 2))
+        if slots is not None:
+            self._need(slots, "slots", _I32, (t,))
+            self._key_value_pages(k_cache, v_cache, q_full.dtype, 1, page_size, rank + rot, rank)
+        self._run("egpt_latent_prep", proj.data_ptr(), splits, int(width), q_plain.data_ptr(), q_full.data_ptr(),
+                  c_weight.data_ptr(), float(eps), self._ptr(cos_sin) if rotary_dim else None, float(magnitude),
+                  int(rotary_dim), self._ptr(slots), self._ptr(k_cache) if slots is not None else None,
+                  self._ptr(v_cache) if slots is not None else None, t, nq, dim, rot, rank, page_size, dt, self._stream())
+
+    def heads_product(self, x, w):
+        with _FirstChoice():
+            return torch.bmm(x, w)
+
+    def sigmoid_gate(self, x, heads, gate, gate_offset, out):
+        t, n = out.shape
+        dt = self._act(out, "out")
+        self._need(out, "out")
+        self._need(x, "x", out.dtype, (heads, t, n // heads) if heads else (t, n))
+        width = gate.shape[-1]
+        splits = self._product(gate, "gate", out.dtype, t, width)
+        if gate_offset < 0 or gate_offset + n > width:
+            raise ValueError(f"gate columns {gate_offset}..{gate_offset + n} lie outside rows of {width} values")
+        self._run("egpt_sigmoid_gate", x.data_ptr(), int(heads), gate.data_ptr(), splits, int(width), int(gate_offset),
+                  out.data_ptr(), t, n, dt, self._stream())
+
+    def window_attention(self, q, out, k_cache, v_cache, block_table, q_start, q_len, kv_len, nq, nkv, dk, dv, page_size,
+                         scale, window, keep_first, sink, max_q_len, max_kv_len):
+        t = q.shape[0]
+        b, width = block_table.shape
+        dt = self._act(q, "q")
+        self._need(q, "q", None, (t, nq * dk))
+        self._need(out, "out", q.dtype, (t, nq * dv))
+        self._key_value_pages(k_cache, v_cache, q.dtype, nkv, page_size, dk, dv)
+        self._need(block_table, "block_table", _I32)
+        for name, v in (("q_start", q_start), ("q_len", q_len), ("kv_len", kv_len)):
+            self._need(v, name, _I32, (b,))
+        if sink is not None:
+            self._need(sink, "sink", _F32, (nq,))
+        if max_kv_len > width * page_size:
+            raise ValueError(f"block table of width {width} cannot hold {max_kv_len} tokens at page size {page_size}")
+        if dk > self.max_window_attention_dim or dv > self.max_window_attention_dim:
+            raise ValueError(f"key size {dk} / value size {dv} is not supported (at most {self.max_window_attention_dim})")
+        self._run("egpt_window_attention", q.data_ptr(), out.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
+                  block_table.data_ptr(), width, q_start.data_ptr(), q_len.data_ptr(), kv_len.data_ptr(), b, t, nq, nkv,
+                  dk, dv, page_size, float(scale), int(window), int(keep_first), self._ptr(sink), dt, self._stream())
 
     def swiglu(self, gate_up, out, row_ss=None, hidden=0, eps=0.0):
         """out = up * silu(gate) for gate_up act [T, 2I] or float32 partial sums [S, T, 2I].  row_ss float32

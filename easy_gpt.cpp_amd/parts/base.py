@@ -42,18 +42,24 @@ class CacheNeed:
 
     window None: every earlier token stays readable.  window W: a token reads only
     the last W tokens (itself included); pages wholly behind that are given back.
+    keep_first F (with a window): a token also reads the first F tokens of its request,
+    whose pages are never given back.
     Mixers with equal needs share a page pool and a block table per request.
     """
 
     tensors: tuple[PagedTensor, ...]
     window: int | None = None
+    keep_first: int = 0
 
     @classmethod
-    def keys_and_values(cls, n_kv_heads: int, head_dim: int, window: int | None = None) -> "CacheNeed":
+    def keys_and_values(cls, n_kv_heads: int, head_dim: int, window: int | None = None,
+                        value_dim: int | None = None, keep_first: int = 0) -> "CacheNeed":
         """Attention's cache: keys [n_kv_heads, page_size, head_dim] per page (a key's features contiguous) and
-        values [n_kv_heads, head_dim, page_size] (a feature's values over the page's tokens contiguous): each the
-        order in which the matrix cores take their operands."""
-        return cls((PagedTensor("k", (n_kv_heads, head_dim), 1), PagedTensor("v", (n_kv_heads, head_dim), 2)), window)
+        values [n_kv_heads, value_dim, page_size] (a feature's values over the page's tokens contiguous; value_dim
+        is head_dim unless given): each the order in which the matrix cores take their operands."""
+        vd = head_dim if value_dim is None else value_dim
+        return cls((PagedTensor("k", (n_kv_heads, head_dim), 1), PagedTensor("v", (n_kv_heads, vd), 2)), window,
+                   int(keep_first) if window else 0)
 
 
 @dataclass(frozen=True)

@@ -3,9 +3,13 @@
 Pre-norm with two residual additions, as the reference's block
 (/root/reference/src/models/block.cpp:23-29): a = x + Mixer(N1(x)); y = a + FF(N2(a)).
 The additions are made in float32 inside the following norm's kernel.
+Parallel with one norm: x = N(h); y = h + Mixer(x) + FF(x).
 """
 from __future__ import annotations
 
+import torch
+
+from .. import kernels
 from .base import Block, PendingNorm, register_part
 
 
@@ -23,4 +27,34 @@ class PreNormBlock(Block):
         return pending.h_after, m                                            # m is added by whoever comes next
 
 
+class ParallelBlock(Block):
+    """One norm whose output both branches read, both added to the stream: x = N(h); y = h + Mixer(x) + FF(x).
+    The two branch outputs go on as one not-yet-added delta: float32 partial sums of both products side by side
+    (the next norm's kernel adds them in float32), or, when a branch returns a rounded tensor, the mixer's output
+    is added to the stream here and the feed-forward's goes on."""
+
+    norm_slots = ("input",)
+
+    def forward(self, h, delta, ctx, cache, state):
+        pending = PendingNorm(h, delta, self.norms["input"])
+        x = pending.materialize()
+        h = pending.h_after
+        a = self.mixer.forward(x, ctx, cache, state)
+        m = self.feed_forward.forward(x, ctx) if self.feed_forward is not None else None
+        if a is None or m is None:
+            return h, (m if a is None else a)
+        if a.dim() == 3 and m.dim() == 3 and a.dtype == m.dtype == torch.float32:
+            return h, torch.cat([a, m], dim=0)
+        kernels.backend().residual_add(h, a)
+        return h, m
+
+
+class ParallelMixerOnlyBlock(ParallelBlock):
+    """The parallel arrangement of a layer that has no feed-forward: y = h + Mixer(N(h))."""
+
+    uses_feed_forward = False
+
+
 register_part("block", "pre_norm", PreNormBlock)
+register_part("block", "parallel", ParallelBlock)
+register_part("block", "parallel_mixer_only", ParallelMixerOnlyBlock)

@@ -18,17 +18,18 @@ from .spec import ParamSpec
 class TokenEmbedding(Embedding):
     graph_safe = True
 
-    def __init__(self, prefix: str, hidden_size: int, vocab_size: int):
+    def __init__(self, prefix: str, hidden_size: int, vocab_size: int, name: str = "weight"):
         self.prefix = prefix
         self.hidden_size = int(hidden_size)
         self.vocab_size = int(vocab_size)
+        self.name = name                   # the table is the tensor `prefix + name`
         self.table: torch.Tensor | None = None
 
     def param_specs(self):
-        return [ParamSpec(self.prefix + "weight", (self.vocab_size, self.hidden_size), role="embedding")]
+        return [ParamSpec(self.prefix + self.name, (self.vocab_size, self.hidden_size), role="embedding")]
 
     def load(self, get, dtype, device):
-        self.table = self._to(get(self.prefix + "weight"), "compute", dtype, device)
+        self.table = self._to(get(self.prefix + self.name), "compute", dtype, device)
 
     def output_matrix(self) -> torch.Tensor:
         return self.table
@@ -42,24 +43,52 @@ class TokenEmbedding(Embedding):
         return out
 
 
+class NormedTokenEmbedding(TokenEmbedding):
+    """x[t, :] = N(E[id_t, :]) with an RMS norm that has one gain for all coordinates (the tensor `prefix + norm_name`):
+    gather, statistics and the product with the gain in one kernel, in float32, written as the residual stream.  The
+    stream of such a model is float32 in steps of any size."""
+
+    def __init__(self, prefix: str, hidden_size: int, vocab_size: int, eps: float, name: str = "weight",
+                 norm_name: str = "norm"):
+        super().__init__(prefix, hidden_size, vocab_size, name)
+        self.eps = float(eps)
+        self.norm_name = norm_name
+        self.gain: torch.Tensor | None = None
+
+    def param_specs(self):
+        return super().param_specs() + [ParamSpec(self.prefix + self.norm_name, (), role="norm_scale", alt_shapes=((1,),))]
+
+    def load(self, get, dtype, device):
+        super().load(get, dtype, device)
+        gain = get(self.prefix + self.norm_name).reshape(1).to(dtype)
+        self.gain = gain.expand(self.hidden_size).to(device).contiguous()
+
+    def forward(self, ctx) -> torch.Tensor:
+        token_ids = ctx.token_ids
+        out = torch.empty((token_ids.shape[0], self.hidden_size), device=token_ids.device, dtype=torch.float32)
+        kernels.backend().embed_rmsnorm(token_ids, self.table, self.gain, self.eps, out)
+        return out
+
+
 class LinearHead(OutputHead):
     graph_safe = True
 
-    def __init__(self, prefix: str, hidden_size: int, vocab_size: int, tied: bool):
+    def __init__(self, prefix: str, hidden_size: int, vocab_size: int, tied: bool, name: str = "weight"):
         self.prefix = prefix
         self.hidden_size = int(hidden_size)
         self.vocab_size = int(vocab_size)
         self.tied = bool(tied)
+        self.name = name                   # the matrix is the tensor `prefix + name`
         self.weight: torch.Tensor | None = None
 
     def param_specs(self):
         if self.tied:
             return []
-        return [ParamSpec(self.prefix + "weight", (self.vocab_size, self.hidden_size))]
+        return [ParamSpec(self.prefix + self.name, (self.vocab_size, self.hidden_size))]
 
     def load(self, get, dtype, device):
         if not self.tied:
-            self.weight = self._to(get(self.prefix + "weight"), "compute", dtype, device)
+            self.weight = self._to(get(self.prefix + self.name), "compute", dtype, device)
 
     def tie(self, matrix: torch.Tensor) -> None:
         if tuple(matrix.shape) != (self.vocab_size, self.hidden_size):
@@ -74,4 +103,5 @@ class LinearHead(OutputHead):
 
 
 register_part("embedding", "token_embedding", TokenEmbedding)
+register_part("embedding", "token_embedding_normed", NormedTokenEmbedding)
 register_part("output_head", "linear_head", LinearHead)

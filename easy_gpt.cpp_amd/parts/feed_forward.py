@@ -19,27 +19,31 @@ class SwiGLU(FeedForward):
     graph_safe = True
     takes_pending_norm = True
 
-    def __init__(self, prefix: str, hidden_size: int, intermediate_size: int, activation: str = "silu"):
+    def __init__(self, prefix: str, hidden_size: int, intermediate_size: int, activation: str = "silu",
+                 names: tuple[str, str, str] = ("gate_proj.weight", "up_proj.weight", "down_proj.weight"),
+                 unrounded: bool = False):
+        """names: the tensors of the gate, up and down matrices behind `prefix`.  unrounded: the output is always
+        float32 partial sums (for an arrangement that adds it to another branch's before anything is rounded)."""
         if activation != "silu":
             raise ValueError(f"activation '{activation}' is not supported by the swiglu feed-forward")
         self.prefix = prefix
         self.hidden_size = int(hidden_size)
         self.intermediate_size = int(intermediate_size)
+        self.names = tuple(names)
+        self.unrounded = bool(unrounded)
         self.w_gate_up = self.w_down = None
 
     def param_specs(self):
         p, h, i = self.prefix, self.hidden_size, self.intermediate_size
-        return [
-            ParamSpec(p + "gate_proj.weight", (i, h)),
-            ParamSpec(p + "up_proj.weight", (i, h)),
-            ParamSpec(p + "down_proj.weight", (h, i)),
-        ]
+        gate, up, down = self.names
+        return [ParamSpec(p + gate, (i, h)), ParamSpec(p + up, (i, h)), ParamSpec(p + down, (h, i))]
 
     def load(self, get, dtype, device):
         p = self.prefix
-        w = torch.cat([get(p + "gate_proj.weight").to(dtype), get(p + "up_proj.weight").to(dtype)], dim=0)
+        gate, up, down = self.names
+        w = torch.cat([get(p + gate).to(dtype), get(p + up).to(dtype)], dim=0)
         self.w_gate_up = w.to(device).contiguous()
-        self.w_down = self._to(get(p + "down_proj.weight"), "compute", dtype, device)
+        self.w_down = self._to(get(p + down), "compute", dtype, device)
 
     def forward(self, x, ctx=None):
         k = kernels.backend()
@@ -48,7 +52,7 @@ class SwiGLU(FeedForward):
         residual = None
 
         def down(act):
-            out = k.product(act, self.w_down, residual=residual)     # else added to the residual stream by the next norm
+            out = k.product(act, self.w_down, unrounded=self.unrounded, residual=residual)     # else added to the residual stream by the next norm
             return None if out is residual else out
 
         if isinstance(x, PendingNorm):

@@ -1,0 +1,188 @@
+"""Attention mixers that treat single heads before the scores: norms per head, a window that keeps the first tokens,
+latent keys and values, a sink in the softmax, an output gate.
+
+Both mixers here run the same three steps through the backend: one product for everything that reads the mixer's
+input, a preparation kernel that norms, rotates and stores into the cache pages, and `window_attention`, the
+attention kernel with separate key and value sizes, window, kept first tokens and sink.
+
+`NormedAttention`: grouped-query attention whose queries and keys are RMS-normed per head with a weight that the
+heads share, whose values are divided by their root mean square before they are cached, and whose window keeps the
+request's first tokens visible: position i sees j <= i if i - j < window or j < keep_first.
+
+`LatentAttention`: every token leaves one latent vector c (RMS-normed, `latent_dim` wide) and one rotated key part
+that all heads share; a head's unrotated key is W_uk c and its value W_uv c.  Only c and the rotated part are cached.
+The scores are computed in the latent space: (q_plain . W_uk c) = ((W_uk^T q_plain) . c), so the query's unrotated
+part is carried into the latent space once per token and head, the cache is read as one key/value head with keys
+[c | rotated part] and values c, and the heads' outputs are carried back with W_uv afterwards.  The softmax's
+denominator holds exp(sink_h) beside the keys' terms; the heads' outputs are multiplied by sigmoid(W_g x).
+"""
+from __future__ import annotations
+
+import torch
+
+from .. import kernels
+from .base import CacheNeed, Mixer, PagedTensor, make_part, register_part
+from .spec import ParamSpec, PartSpec
+
+
+def _window(window) -> int | None:
+    return int(window) if window else None
+
+
+class NormedAttention(Mixer):
+    graph_safe = True
+
+    def __init__(self, prefix: str, hidden_size: int, n_heads: int, n_kv_heads: int, key_dim: int, value_dim: int,
+                 scale: float, eps: float, window: int | None = None, keep_first: int = 0, norm_queries_keys: bool = True,
+                 norm_values: bool = False, names: dict | None = None):
+        """names: tensor names behind `prefix` of q, k, v, o and of the weights q_norm, k_norm."""
+        if n_heads % n_kv_heads:
+            raise ValueError(f"n_heads ({n_heads}) must be a multiple of n_kv_heads ({n_kv_heads})")
+        widest = kernels.KernelBackend.max_window_attention_dim
+        if not (0 < int(key_dim) <= widest and 0 < int(value_dim) <= widest):
+            raise ValueError(f"key size {key_dim} / value size {value_dim} is not supported by the attention kernel (1 to {widest})")
+        self.prefix, self.hidden_size = prefix, int(hidden_size)
+        self.n_heads, self.n_kv_heads = int(n_heads), int(n_kv_heads)
+        self.key_dim, self.value_dim = int(key_dim), int(value_dim)
+        self.scale, self.eps = float(scale), float(eps)
+        self.window = _window(window)
+        self.keep_first = int(keep_first) if self.window else 0
+        self.norm_queries_keys, self.norm_values = bool(norm_queries_keys), bool(norm_values)
+        self.names = dict(q="q_proj.weight", k="k_proj.weight", v="v_proj.weight", o="o_proj.weight",
+                          q_norm="q_norm.weight", k_norm="k_norm.weight")
+        self.names.update(names or {})
+        self.w_qkv = self.w_o = self.q_weight = self.k_weight = None
+
+    def cache_need(self):
+        return CacheNeed.keys_and_values(self.n_kv_heads, self.key_dim, self.window, self.value_dim, self.keep_first)
+
+    def param_specs(self):
+        p, h, n = self.prefix, self.hidden_size, self.names
+        specs = [
+            ParamSpec(p + n["q"], (self.n_heads * self.key_dim, h)),
+            ParamSpec(p + n["k"], (self.n_kv_heads * self.key_dim, h)),
+            ParamSpec(p + n["v"], (self.n_kv_heads * self.value_dim, h)),
+            ParamSpec(p + n["o"], (h, self.n_heads * self.value_dim)),
+        ]
+        if self.norm_queries_keys:
+            specs += [ParamSpec(p + n["q_norm"], (self.key_dim,), role="norm_scale"),
+                      ParamSpec(p + n["k_norm"], (self.key_dim,), role="norm_scale")]
+        return specs
+
+    def load(self, get, dtype, device):
+        p, n = self.prefix, self.names
+        w = torch.cat([get(p + n[x]).to(dtype) for x in "qkv"], dim=0)      # one product serves all three
+        self.w_qkv = w.to(device).contiguous()
+        self.w_o = self._to(get(p + n["o"]), "compute", dtype, device)
+        if self.norm_queries_keys:
+            self.q_weight = self._to(get(p + n["q_norm"]), "compute", dtype, device)
+            self.k_weight = self._to(get(p + n["k_norm"]), "compute", dtype, device)
+
+    def forward(self, x, ctx, cache, state=None):
+        k = kernels.backend()
+        t = x.shape[0]
+        proj = k.product(x, self.w_qkv, unrounded=True)
+        q = torch.empty((t, self.n_heads * self.key_dim), dtype=x.dtype, device=x.device)
+        k.head_norm_store(proj, q, self.q_weight, self.k_weight, self.eps, self.norm_values,
+                          cache.slots if cache.writes else None, cache.k, cache.v, self.n_heads, self.n_kv_heads,
+                          self.key_dim, self.value_dim, cache.page_size)
+        attn = torch.empty((t, self.n_heads * self.value_dim), dtype=x.dtype, device=x.device)
+        k.window_attention(q, attn, cache.k, cache.v, cache.block_table, ctx.q_start, ctx.q_len, ctx.kv_len,
+                           self.n_heads, self.n_kv_heads, self.key_dim, self.value_dim, cache.page_size, self.scale,
+                           self.window or 0, self.keep_first, None, ctx.max_q_len, ctx.max_kv_len)
+        return k.product(attn, self.w_o, unrounded=True)
+
+
+class LatentAttention(Mixer):
+    graph_safe = True
+
+    def __init__(self, prefix: str, hidden_size: int, n_heads: int, plain_dim: int, rotated_dim: int, value_dim: int,
+                 latent_dim: int, scale: float, eps: float, position: PartSpec, window: int | None = None,
+                 sink: bool = False, gated: bool = False, names: dict | None = None):
+        """plain_dim / rotated_dim: a head's unrotated and rotated query/key places (a query head is laid out
+        [plain | rotated]); latent_dim: the width of the cached latent.  names: tensor names behind `prefix` of q, down
+        (rows: latent, then the shared rotated key), down_norm, up_k, up_v, sink, gate, o."""
+        widest = kernels.KernelBackend.max_window_attention_dim
+        if not 0 < int(latent_dim) + int(rotated_dim) <= widest:
+            raise ValueError(f"latent size {latent_dim} + rotated size {rotated_dim} is not supported by the attention "
+                             f"kernel (at most {widest})")
+        self.prefix, self.hidden_size = prefix, int(hidden_size)
+        self.n_heads = int(n_heads)
+        self.plain_dim, self.rotated_dim = int(plain_dim), int(rotated_dim)
+        self.value_dim, self.latent_dim = int(value_dim), int(latent_dim)
+        self.scale, self.eps = float(scale), float(eps)
+        self.window = _window(window)
+        self.has_sink, self.gated = bool(sink), bool(gated)
+        self.position = make_part("position_encoding", position, head_dim=max(self.rotated_dim, 2))
+        self.names = dict(q="q", down="down", down_norm="down_norm", up_k="up_k", up_v="up_v", sink="sink", gate="gate", o="o")
+        self.names.update(names or {})
+        self.q_width = self.n_heads * (self.plain_dim + self.rotated_dim)
+        self.down_width = self.latent_dim + self.rotated_dim
+        self.out_width = self.n_heads * self.value_dim
+        self.w_in = self.w_up_k = self.w_up_v = self.w_o = self.c_weight = self.sink = None
+
+    def cache_need(self):
+        # one key/value head: keys [latent | rotated part], values the latent, transposed within a page
+        return CacheNeed((PagedTensor("k", (1, self.latent_dim + self.rotated_dim), 1),
+                          PagedTensor("v", (1, self.latent_dim), 2)), self.window)
+
+    def param_specs(self):
+        p, h, n = self.prefix, self.hidden_size, self.names
+        specs = [
+            ParamSpec(p + n["q"], (self.q_width, h)),
+            ParamSpec(p + n["down"], (self.down_width, h)),
+            ParamSpec(p + n["down_norm"], (self.latent_dim,), role="norm_scale"),
+            ParamSpec(p + n["up_k"], (self.n_heads * self.plain_dim, self.latent_dim)),
+            ParamSpec(p + n["up_v"], (self.out_width, self.latent_dim)),
+            ParamSpec(p + n["o"], (h, self.out_width)),
+        ]
+        if self.has_sink:
+            specs.append(ParamSpec(p + n["sink"], (self.n_heads,), role="bias", dtype="float32"))
+        if self.gated:
+            specs.append(ParamSpec(p + n["gate"], (self.out_width, h)))
+        return specs + self.position.param_specs()
+
+    def load(self, get, dtype, device):
+        p, n = self.prefix, self.names
+        rows = [get(p + n["q"]).to(dtype), get(p + n["down"]).to(dtype)]
+        if self.gated:
+            rows.append(get(p + n["gate"]).to(dtype))
+        self.w_in = torch.cat(rows, dim=0).to(device).contiguous()          # one product for all that reads x
+        self.w_up_k = self._to(get(p + n["up_k"]), "compute", dtype, device).view(self.n_heads, self.plain_dim, self.latent_dim)
+        w_up_v = self._to(get(p + n["up_v"]), "compute", dtype, device).view(self.n_heads, self.value_dim, self.latent_dim)
+        self.w_up_v = w_up_v.transpose(1, 2).contiguous()                    # [heads, latent, value]
+        self.w_o = self._to(get(p + n["o"]), "compute", dtype, device)
+        self.c_weight = self._to(get(p + n["down_norm"]), "compute", dtype, device)
+        if self.has_sink:
+            self.sink = get(p + n["sink"]).to(torch.float32).to(device).contiguous()
+        self.position.load(get, dtype, device)
+
+    def forward(self, x, ctx, cache, state=None):
+        k = kernels.backend()
+        t, nh, rank, rot = x.shape[0], self.n_heads, self.latent_dim, self.rotated_dim
+        proj = k.product(x, self.w_in, unrounded=True)
+        q_plain = torch.empty((t, nh, self.plain_dim), dtype=x.dtype, device=x.device)
+        q_full = torch.empty((t, nh, rank + rot), dtype=x.dtype, device=x.device)
+        rotary = self.position.rotary(x.device)
+        cos_sin = self.position.table(ctx) if rotary is not None else None
+        k.latent_prep(proj, q_plain, q_full, self.c_weight, self.eps, cos_sin, getattr(self.position, "magnitude", 1.0),
+                      rotary[1] if rotary is not None else 0, cache.slots if cache.writes else None, cache.k, cache.v,
+                      nh, self.plain_dim, rot, rank, cache.page_size)
+        # the queries' unrotated parts carried into the latent space, head by head
+        q_full[:, :, :rank].copy_(k.heads_product(q_plain.transpose(0, 1), self.w_up_k).transpose(0, 1))
+        o_latent = torch.empty((t, nh * rank), dtype=x.dtype, device=x.device)
+        k.window_attention(q_full.view(t, nh * (rank + rot)), o_latent, cache.k, cache.v, cache.block_table, ctx.q_start,
+                           ctx.q_len, ctx.kv_len, nh, 1, rank + rot, rank, cache.page_size, self.scale, self.window or 0,
+                           0, self.sink, ctx.max_q_len, ctx.max_kv_len)
+        # and the heads' outputs carried back: [heads, T, value]
+        o = k.heads_product(o_latent.view(t, nh, rank).transpose(0, 1), self.w_up_v)
+        if self.gated:
+            heads_out = torch.empty((t, self.out_width), dtype=x.dtype, device=x.device)
+            k.sigmoid_gate(o, nh, proj, self.q_width + self.down_width, heads_out)
+        else:
+            heads_out = o.transpose(0, 1).reshape(t, self.out_width)
+        return k.product(heads_out, self.w_o, unrounded=True)
+
+
+register_part("mixer", "normed_attention", NormedAttention)
+register_part("mixer", "latent_attention", LatentAttention)

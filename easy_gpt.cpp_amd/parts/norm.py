@@ -44,4 +44,22 @@ class RMSNorm(Norm):
         return out
 
 
+class ScalarRMSNorm(RMSNorm):
+    """RMS norm with one gain for all coordinates: y = x / sqrt(mean(x^2) + eps) * g.  The gain is a tensor with a
+    single number (`prefix + name`); on the device it is repeated over the width, so the kernels of the norm with a
+    weight per coordinate run it, and parts that fold a norm into their first kernel see an ordinary weight."""
+
+    def __init__(self, prefix: str, hidden_size: int, eps: float, name: str = "weight"):
+        super().__init__(prefix, hidden_size, eps)
+        self.name = name
+
+    def param_specs(self):
+        return [ParamSpec(self.prefix + self.name, (), role="norm_scale", alt_shapes=((1,),))]
+
+    def load(self, get, dtype, device):
+        gain = get(self.prefix + self.name).reshape(1).to(dtype)
+        self.weight = gain.expand(self.hidden_size).to(device).contiguous()
+
+
 register_part("norm", "rmsnorm", RMSNorm)
+register_part("norm", "rmsnorm_scalar", ScalarRMSNorm)

@@ -8,6 +8,8 @@ queries and keys, never to values.
 """
 from __future__ import annotations
 
+import math
+
 import torch
 
 from .. import kernels
@@ -52,6 +54,52 @@ class RotaryHalfSplit(PositionEncoding):
         return ctx.shared[key]
 
 
+class RotaryInterleaved(RotaryHalfSplit):
+    """Rotation of neighbouring places: the pair (2i, 2i + 1) of the first `rotary_dim` places turns by
+    position * f_i, f_i = theta^(-2i / rotary_dim).  The kernels of the mixers that use it rotate from the step's
+    table of cosines and sines (`table`) and multiply both by `magnitude`.
+
+    scaling = {factor, original, fast, slow} stretches the slow frequencies for contexts beyond the `original`
+    length (YaRN): with dim(t) = rotary_dim * ln(original / (2 pi t)) / (2 ln theta), lo = max(floor(dim(fast)), 0),
+    hi = min(ceil(dim(slow)), rotary_dim - 1) and ramp_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1), the
+    frequency is f_i / factor * ramp_i + f_i * (1 - ramp_i), and magnitude = 0.1 * ln(factor) + 1."""
+
+    def __init__(self, prefix: str, head_dim: int, theta: float, rotary_dim: int | None = None, scaling=None, **_):
+        super().__init__(prefix, head_dim, theta, rotary_dim)
+        self.scaling = dict(scaling) if scaling else None
+        self.magnitude = 1.0
+        if self.scaling:
+            for key in ("factor", "original", "fast", "slow"):
+                if not float(self.scaling.get(key, 0)) > 0:
+                    raise ValueError(f"rotation scaling needs a positive '{key}'")
+            self.magnitude = 0.1 * math.log(float(self.scaling["factor"])) + 1.0
+
+    def inv_freq_host(self) -> torch.Tensor:
+        d = self.rotary_dim
+        i = torch.arange(0, d // 2, dtype=torch.float64)
+        f = torch.pow(torch.tensor(self.theta, dtype=torch.float64), -2.0 * i / float(d))
+        if self.scaling:
+            sc = self.scaling
+            factor, original = float(sc["factor"]), float(sc["original"])
+
+            def place_of(turns: float) -> float:
+                return d * math.log(original / (2.0 * math.pi * turns)) / (2.0 * math.log(self.theta))
+
+            lo = max(math.floor(place_of(float(sc["fast"]))), 0)
+            hi = min(math.ceil(place_of(float(sc["slow"]))), d - 1)
+            ramp = torch.clamp((i - lo) / max(hi - lo, 0.001), 0.0, 1.0)
+            f = f / factor * ramp + f * (1.0 - ramp)
+        return f.to(torch.float32)
+
+    def table(self, ctx):
+        sc = tuple(sorted(self.scaling.items())) if self.scaling else None
+        key = ("rope_table_interleaved", self.theta, self.rotary_dim, sc)
+        if key not in ctx.shared:
+            inv_freq, _ = self.rotary(ctx.positions.device)
+            ctx.shared[key] = kernels.backend().rope_table(ctx.positions, inv_freq)
+        return ctx.shared[key]
+
+
 class NoPosition(PositionEncoding):
     """No position information enters the mixer."""
 
@@ -68,4 +116,5 @@ class NoPosition(PositionEncoding):
 
 
 register_part("position_encoding", "rope_half_split", RotaryHalfSplit)
+register_part("position_encoding", "rope_interleaved", RotaryInterleaved)
 register_part("position_encoding", "none", NoPosition)

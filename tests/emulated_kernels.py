@@ -54,7 +54,7 @@ class EmulatedKernels(KernelBackend):
         out.copy_(y.to(out.dtype))
 
     def qkv_rope_store(self, qkv, bias, positions, inv_freq, rotary_dim, slots, k_cache, v_cache, nq, nkv, hd,
-                       page_size, out=None):
+                       page_size, out=None, cos_sin=None):
         src = _whole(qkv)
         qkv = src if out is None else out
         t = qkv.shape[0]
@@ -101,6 +101,99 @@ class EmulatedKernels(KernelBackend):
                     sc = (keys @ q_all[s + i, h]) * scale
                     pr = torch.softmax(sc, dim=0)
                     out[s + i, h * hd : (h + 1) * hd] = (pr @ vals).to(out.dtype)
+
+    def rope_table(self, positions, inv_freq):
+        ang = (positions.to(torch.float32)[:, None] * inv_freq[None, :]).to(F64)
+        return torch.stack([torch.cos(ang), torch.sin(ang)], dim=-1).to(torch.float32)
+
+    def embed_rmsnorm(self, token_ids, table, weight, eps, out):
+        x = table[token_ids.long()].to(F64)
+        inv = 1.0 / torch.sqrt((x * x).mean(-1, keepdim=True) + eps)
+        out.copy_((x * inv * weight.to(F64)).to(out.dtype))
+
+    @staticmethod
+    def _store(k_cache, v_cache, slots, page_size, keys, values):
+        page, off = (slots // page_size).long(), (slots % page_size).long()
+        for i in range(keys.shape[0]):
+            k_cache[page[i], :, off[i], :] = keys[i].to(k_cache.dtype)
+            v_cache[page[i], :, :, off[i]] = values[i].to(v_cache.dtype)
+
+    def head_norm_store(self, proj, q_out, q_weight, k_weight, eps, norm_values, slots, k_cache, v_cache, nq, nkv, dk, dv,
+                        page_size):
+        x = _whole(proj).to(F64)
+        t = x.shape[0]
+        unit = lambda a: a / torch.sqrt((a * a).mean(-1, keepdim=True) + eps)
+        q = x[:, : nq * dk].view(t, nq, dk)
+        k = x[:, nq * dk : (nq + nkv) * dk].view(t, nkv, dk)
+        v = x[:, (nq + nkv) * dk :].view(t, nkv, dv)
+        if q_weight is not None:
+            q = unit(q) * q_weight.to(F64)
+        if k_weight is not None:
+            k = unit(k) * k_weight.to(F64)
+        if norm_values:
+            v = unit(v)
+        q_out.copy_(q.reshape(t, nq * dk).to(q_out.dtype))
+        if slots is not None:
+            self._store(k_cache, v_cache, slots, page_size, k, v)
+
+    def latent_prep(self, proj, q_plain, q_full, c_weight, eps, cos_sin, magnitude, rotary_dim, slots, k_cache, v_cache,
+                    nq, dim, rot, rank, page_size):
+        x = _whole(proj).to(F64)
+        t = x.shape[0]
+        q = x[:, : nq * (dim + rot)].view(t, nq, dim + rot)
+        base = nq * (dim + rot)
+        c, shared = x[:, base : base + rank], x[:, base + rank : base + rank + rot]
+        c = c / torch.sqrt((c * c).mean(-1, keepdim=True) + eps) * c_weight.to(F64)
+
+        def turn(a):                                   # a [..., T, rot] with T second to last
+            a = a.clone()
+            if rotary_dim:
+                cs = cos_sin.to(F64) * magnitude
+                co, si = cs[:, :, 0], cs[:, :, 1]
+                u, w = a[..., 0:rotary_dim:2].clone(), a[..., 1:rotary_dim:2].clone()
+                a[..., 0:rotary_dim:2] = u * co - w * si
+                a[..., 1:rotary_dim:2] = w * co + u * si
+            return a
+
+        q_plain.copy_(q[..., :dim].to(q_plain.dtype))
+        q_full[..., rank:] = turn(q[..., dim:].transpose(0, 1)).transpose(0, 1).to(q_full.dtype)
+        if slots is not None:
+            keys = torch.cat([c, turn(shared)], dim=-1).view(t, 1, rank + rot)
+            self._store(k_cache, v_cache, slots, page_size, keys, c.view(t, 1, rank))
+
+    def heads_product(self, x, w):
+        return torch.bmm(x.to(F64), w.to(F64)).to(x.dtype)
+
+    def sigmoid_gate(self, x, heads, gate, gate_offset, out):
+        t, n = out.shape
+        g = _whole(gate)[:, gate_offset : gate_offset + n].to(F64)
+        xx = x.to(F64)
+        if heads:
+            xx = xx.transpose(0, 1).reshape(t, n)
+        out.copy_((xx * torch.sigmoid(g)).to(out.dtype))
+
+    def window_attention(self, q, out, k_cache, v_cache, block_table, q_start, q_len, kv_len, nq, nkv, dk, dv, page_size,
+                         scale, window, keep_first, sink, max_q_len, max_kv_len):
+        group = nq // nkv
+        q_all = q.view(q.shape[0], nq, dk).to(F64)
+        for b in range(q_start.shape[0]):
+            s, n, kv = int(q_start[b]), int(q_len[b]), int(kv_len[b])
+            for i in range(n):
+                p = kv - n + i
+                lo = max(0, p - window + 1) if window else 0
+                js = torch.cat([torch.arange(0, min(keep_first, lo)), torch.arange(lo, p + 1)])
+                pages = block_table[b, (js // page_size)].long()
+                assert (pages >= 0).all(), "attention would read a page that was given back"
+                offs = (js % page_size).long()
+                for h in range(nq):
+                    kh = h // group
+                    keys = k_cache[pages, kh, offs, :].to(F64)
+                    vals = v_cache[pages, kh, :, offs].to(F64)
+                    sc = (keys @ q_all[s + i, h]) * scale
+                    m = sc.max() if sink is None else torch.maximum(sc.max(), sink[h].to(F64))
+                    e = torch.exp(sc - m)
+                    denom = e.sum() + (torch.exp(sink[h].to(F64) - m) if sink is not None else 0.0)
+                    out[s + i, h * dv : (h + 1) * dv] = ((e / denom) @ vals).to(out.dtype)
 
     def swiglu(self, gate_up, out):
         gate_up = _whole(gate_up)

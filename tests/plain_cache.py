@@ -182,10 +182,11 @@ class PlainCacheManager:
             # the next token (position num_tokens) reads keys j > num_tokens - window
             first_needed = rc.num_tokens - need.window + 1
             dead_pages = max(0, first_needed) // self.page_size   # pages wholly below first_needed
-            gone = [p for p in table[:dead_pages] if p >= 0]
+            kept = _ceil_div(getattr(need, "keep_first", 0) or 0, self.page_size)   # pages that hold a kept first token
+            gone = [p for p in table[kept:dead_pages] if p >= 0]
             if gone:
                 pool.give_back(gone)
-                for i in range(dead_pages):
+                for i in range(kept, dead_pages):
                     table[i] = -1
                 rc.version += 1
 
