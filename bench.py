@@ -372,6 +372,79 @@ def decode_seconds(engine, sampler, rids, last, warmup: int, steps: int, no_look
     return sec, (between[len(between) // 2] if between else sec / steps)
 
 
+# ---------------------------------------------------------------------------------- another design beside the closest model
+# `--design pekasun`: prefill and decode of the Pekasun design at layer sizes that resemble a real model's, beside the
+# Qwen2 model of the same width, depth, heads, inner width and vocabulary (random weights on both sides).  Four layers
+# each: latent attention and windowed attention in turn.  (label, width, inner width, heads, kv heads, head size,
+# latent width, rotated part, window)
+DESIGN_SIZES = (
+    ("w896", 896, 4864, 14, 2, 64, 128, 32, 1024),
+    ("w2048", 2048, 8192, 16, 4, 128, 192, 64, 2048),
+)
+DESIGN_LAYERS, DESIGN_VOCAB, DESIGN_BATCHES = 4, 32768, (1, 8, 64)
+
+
+def pekasun_config(width, inner, heads, kv_heads, hd, rank, rot, window) -> dict:
+    latent = {"type": "latent_attention", "mlp": {"kind": "dense", "ff": inner},
+              "mixer": {"heads": heads, "dim": hd, "rot_dim": rot, "vdim": hd, "kv_rank": rank, "scale": (hd + rot) ** -0.5,
+                        "mask": {"size": window},
+                        "rot": {"base": 10000.0, "dims": rot,
+                                "scaling": {"factor": 4.0, "original": 4096, "fast": 32.0, "slow": 1.0}}}}
+    plain = {"type": "attention", "mlp": {"kind": "dense", "ff": inner},
+             "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": hd, "vdim": hd, "scale": hd ** -0.5,
+                       "mask": {"size": window, "keep_first": 4}}}
+    return {"architecture": "Pekasun", "vocab": DESIGN_VOCAB, "width": width, "norm": {"eps": 1e-6},
+            "layers": [latent, plain] * (DESIGN_LAYERS // 2)}
+
+
+def design_comparison(args) -> dict:
+    import torch
+
+    from easy_gpt.cpp_amd.engine import Engine
+    from easy_gpt.cpp_amd.engine.engine import load_random_model
+    from easy_gpt.cpp_amd.sampling import Sampler
+
+    g = torch.Generator().manual_seed(0)
+    prefix, points = 2048, {}
+    for label, width, inner, heads, kv_heads, hd, rank, rot, window in DESIGN_SIZES:
+        models = {
+            "pekasun": pekasun_config(width, inner, heads, kv_heads, hd, rank, rot, window),
+            "qwen2": dict(QWEN25_05B, hidden_size=width, intermediate_size=inner, num_attention_heads=heads,
+                          num_key_value_heads=kv_heads, head_dim=hd, num_hidden_layers=DESIGN_LAYERS, vocab_size=DESIGN_VOCAB,
+                          tie_word_embeddings=False),
+        }
+        for which, cfg in models.items():
+            model = load_random_model(cfg, seed=0, dtype=args.dtype, device="cuda:0")
+            room = max(DESIGN_BATCHES) * (prefix + 64 + FURTHER_WARMUP + FURTHER_STEPS) + FILL_TOKENS
+            engine = Engine(model, page_size=args.page_size, max_tokens=room, max_requests=max(DESIGN_BATCHES) + 2,
+                            tune_products=not args.no_tune)
+            sampler = Sampler(engine.device)
+            sec = prefill_seconds(engine, DESIGN_VOCAB, PREFILL_TOKENS, g, reps=5)
+            points[f"{label}_{which}_prefill_tokens_per_s"] = round(PREFILL_TOKENS / sec, 1)
+            points[f"{label}_{which}_prefill_ms"] = round(sec * 1e3, 3)
+            for batch in DESIGN_BATCHES:
+                rids, last = fill_requests(engine, sampler, DESIGN_VOCAB, prefix, batch, g)
+                sec, between = decode_seconds(engine, sampler, rids, last, FURTHER_WARMUP, FURTHER_STEPS)
+                for rid in rids:
+                    engine.finish(rid)
+                points[f"{label}_{which}_decode_b{batch}_ms_per_step"] = round(between * 1e3, 4)
+                points[f"{label}_{which}_decode_b{batch}_tokens_per_s"] = round(batch / between, 1)
+            print(f"[bench] {label} {which} done", file=sys.stderr, flush=True)
+            del engine, sampler, model
+            torch.cuda.empty_cache()
+    first = DESIGN_SIZES[0][0]
+    return {
+        "metric": "decode tokens/s of the Pekasun design at batch 8 behind 2,048 tokens (4 layers of width 896)",
+        "value": points[f"{first}_pekasun_decode_b8_tokens_per_s"], "unit": "tokens/s", "n_gpus": 1,
+        "higher_is_better": True, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+        "data": "synthetic: uniform-random token ids, random weights N(0, 0.02) from seed 0",
+        "config": {"layers": DESIGN_LAYERS, "vocab": DESIGN_VOCAB, "prefix": prefix, "prefill_tokens": PREFILL_TOKENS,
+                   "sizes": {s[0]: dict(zip(("width", "inner", "heads", "kv_heads", "head", "latent", "rotated", "window"), s[1:]))
+                             for s in DESIGN_SIZES}},
+        "points": points,
+    }
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -402,12 +475,18 @@ def main() -> int:
     ap.add_argument("--no-lookahead", action="store_true",
                     help="wait for a step's tokens on the host before the next step is launched (the scheduler with --serve, "
                          "the decode loop otherwise)")
+    ap.add_argument("--design", default=None, choices=["pekasun"],
+                    help="instead of the record: prefill and decode of that design at a few layer sizes beside the Qwen2 "
+                         "model of equal sizes")
     ap.add_argument("--direct-loop", action="store_true",
                     help="decode with the engine's step function in a loop of the benchmark's own instead of Scheduler.step")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU: this engine has no multi-GPU path, --gpus {args.gpus} is not run")
         return 2
+    if args.design:
+        print(json.dumps(design_comparison(args)), flush=True)
+        return 0
     global FULL_LAYERS, PREFIX, CONTEXT
     base, name = dict(QWEN25_05B), "Qwen2.5-0.5B"
     if args.shape != "0.5b":
