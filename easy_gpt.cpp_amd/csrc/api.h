@@ -153,6 +153,15 @@ int egpt_window_attention(const void* q, void* out, const void* k_cache, const v
                           int table_width, const int32_t* q_start, const int32_t* q_len, const int32_t* kv_len,
                           int n_seqs, int n_tokens, int nq, int nkv, int dk, int dv, int page_size, float scale,
                           int window, int keep_first, const float* sink, int dtype, void* stream);
+// The same on the matrix cores: dk a multiple of 4 (float32) or 8 (bfloat16), dv a multiple of 16 up to 256, page_size a
+// multiple of 16.  row_tiles: 4 (workgroups of 64 rows, for prompt portions) or 1 (16 rows, for single tokens).  With
+// n_splits > 1 the chunks of keys of a workgroup's rows are dealt over as many workgroups, whose results part_o
+// [n_splits][n_tokens][nq][dv] and part_ml [n_splits][n_tokens][nq][2] (float32) a second kernel folds.
+int egpt_window_attention_tiled(const void* q, void* out, float* part_o, float* part_ml, const void* k_cache,
+                                const void* v_cache, const int32_t* block_table, int table_width, const int32_t* q_start,
+                                const int32_t* q_len, const int32_t* kv_len, int n_seqs, int n_tokens, int nq, int nkv,
+                                int dk, int dv, int page_size, float scale, int window, int keep_first, const float* sink,
+                                int n_splits, int row_tiles, int dtype, void* stream);
 // scratch: n_rows * 32 floats followed by n_rows * 32 int32 (two-stage search for wide vocabularies), or null.
 int egpt_argmax(const float* logits, int32_t* out, void* scratch, int n_rows, int vocab, void* stream);
 // egpt_argmax for callers that cannot allocate device memory and have no workspace to pass (code under graph

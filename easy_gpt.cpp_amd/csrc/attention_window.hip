@@ -149,6 +149,372 @@ __global__ __launch_bounds__(64 * kSimpleWaves) void window_attention_simple_ker
     }
 }
 
+
+// ---------------------------------------------------------------------------------------------- on the matrix cores
+// The same attention for key sizes that are multiples of 16 bytes' worth of elements, value sizes that are multiples
+// of 16 up to 256, and page sizes that are multiples of 16.  Rows are (token, query head) pairs of one key/value
+// head's group, 16 to a wavefront; the scores are computed transposed, S^T[key, row] = K[key, :] . Q[row, :], so that a
+// lane holds scores of one row, the row's statistics are per-lane scalars and the probabilities are the second
+// product's operand as they lie in registers: O^T[feature, row] += V^T[feature, key] . P^T[key, row].
+//   bfloat16: v_mfma_f32_16x16x32_bf16, a lane's 16 bytes of an operand are 8 features (or 8 keys);
+//   float32:  v_mfma_f32_16x16x4_f32 (float32 operands and accumulation), a lane's 16 bytes are 4 features (or 4 keys).
+// A workgroup of RT wavefronts takes 16 * RT rows of one request and key/value head and walks the chunks of KT keys
+// that any of its rows can see: those that hold kept first tokens, then those of the window.  A chunk's keys and values
+// are staged through LDS and shared by the wavefronts; the queries lie in LDS too, so the key size is a run-time
+// number (the value size, which sizes the accumulators, is a template parameter in steps).  With n_splits > 1 the
+// chunks of a workgroup's rows are dealt over as many workgroups (grid z), which leave unnormalised results
+// part_o [split][token][head][dv] and (maximum, sum) part_ml [split][token][head][2] that window_attention_fold_kernel
+// combines; that kernel also adds the sink.  With one split the kernel finishes the rows itself.
+typedef __attribute__((ext_vector_type(8))) __bf16 w_bf16x8;
+typedef __attribute__((ext_vector_type(4))) float w_f32x4;
+typedef __attribute__((ext_vector_type(4))) unsigned int w_u32x4;
+typedef __attribute__((ext_vector_type(2))) unsigned int w_u32x2;
+
+template <typename T>
+__device__ __forceinline__ w_f32x4 matrix_piece(const w_u32x4& a, const w_u32x4& b, w_f32x4 acc) {
+    if constexpr (sizeof(T) == 2) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(w_bf16x8, a), __builtin_bit_cast(w_bf16x8, b), acc,
+                                                       0, 0, 0);
+    } else {
+        const w_f32x4 av = __builtin_bit_cast(w_f32x4, a), bv = __builtin_bit_cast(w_f32x4, b);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(av[i], bv[i], acc, 0, 0, 0);
+        return acc;
+    }
+}
+
+// Before accumulators are read behind a loop whose trip count is known only at run time: the wait between a matrix
+// instruction and the read of its result is counted in instructions along the code, and sixteen idle cycles cover
+// the longest instruction used here whatever path was taken.
+__device__ __forceinline__ void matrix_results_ready() {
+    __builtin_amdgcn_sched_barrier(0);
+    asm volatile("s_nop 15");
+    __builtin_amdgcn_sched_barrier(0);
+}
+
+template <typename T>
+__device__ __forceinline__ void store_four(T* dst, float a, float b, float c, float d) {
+    if constexpr (sizeof(T) == 2) {
+        uint2 packed;
+        packed.x = f32_to_bf16_bits(a) | (static_cast<uint32_t>(f32_to_bf16_bits(b)) << 16);
+        packed.y = f32_to_bf16_bits(c) | (static_cast<uint32_t>(f32_to_bf16_bits(d)) << 16);
+        *reinterpret_cast<uint2*>(dst) = packed;
+    } else {
+        *reinterpret_cast<float4*>(dst) = float4{a, b, c, d};
+    }
+}
+
+struct WindowArgs {
+    const void* q;
+    void* out;
+    float* part_o;
+    float* part_ml;
+    const void* k_cache;
+    const void* v_cache;
+    const int32_t* block_table;
+    const int32_t* q_start;
+    const int32_t* q_len;
+    const int32_t* kv_len;
+    const float* sink;
+    int table_width, n_seqs, n_tokens, nq, nkv, dk, dv, page_size, window, keep_first, n_splits;
+    float scale;
+};
+
+template <typename T, int DT, int RT>
+__global__ __launch_bounds__(64 * RT) void window_attention_tiled_kernel(WindowArgs a) {
+    constexpr int E = 16 / sizeof(T);             // elements in 16 bytes
+    constexpr int KT = sizeof(T) == 2 ? 64 : 32;  // keys per chunk
+    constexpr int NKT = KT / 16;                  // tiles of 16 keys in a chunk
+    constexpr int PF = 4 * E;                     // features (or keys) that one matrix_piece sums over
+    constexpr int NP = KT / PF;                   // pieces of a chunk's keys
+    constexpr int ROWS = 16 * RT, THREADS = 64 * RT;
+    constexpr int VROW = KT + E;                  // padded LDS row of values (elements)
+    extern __shared__ __attribute__((aligned(16))) unsigned char window_smem[];
+    const T* __restrict__ q = static_cast<const T*>(a.q);
+    const T* __restrict__ k_cache = static_cast<const T*>(a.k_cache);
+    const T* __restrict__ v_cache = static_cast<const T*>(a.v_cache);
+    const int dk = a.dk, dv = a.dv, nq = a.nq, nkv = a.nkv, page_size = a.page_size, window = a.window;
+    const int n_pieces = (dk + PF - 1) / PF;
+    const int krow = n_pieces * PF + E;           // padded LDS row of keys and of queries
+    T* q_s = reinterpret_cast<T*>(window_smem);
+    T* k_s = q_s + ROWS * krow;
+    T* v_s = k_s + KT * krow;
+
+    const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+    const int lj = lane % 16, lg = lane / 16;
+    const int kh = blockIdx.y;
+    const int group_size = nq / nkv;
+
+    int b = 0, grp = blockIdx.x;
+    for (; b < a.n_seqs; ++b) {
+        const int groups = (a.q_len[b] * group_size + ROWS - 1) / ROWS;
+        if (grp < groups) break;
+        grp -= groups;
+    }
+    if (b >= a.n_seqs) return;
+    const int n = a.q_len[b], kv = a.kv_len[b], qs = a.q_start[b];
+    const int rows = n * group_size;
+    const int32_t* table = a.block_table + static_cast<size_t>(b) * a.table_width;
+
+    // the workgroup's rows and the chunks of keys that they can see
+    const int blk_first = grp * ROWS, blk_last = min(rows, blk_first + ROWS) - 1;
+    const int p_max = kv - n + blk_last / group_size;
+    const int p_min = kv - n + blk_first / group_size;
+    const int lo_blk = window > 0 ? max(0, p_min - window + 1) : 0;
+    const int t_begin = lo_blk / KT, t_end = p_max / KT + 1;
+    const int keep = window > 0 ? min(a.keep_first, lo_blk) : 0;     // kept first tokens below the window
+    const int kept_chunks = min((keep + KT - 1) / KT, t_begin);
+    const int n_chunks = kept_chunks + (t_end - t_begin);
+    const int per_split = (n_chunks + a.n_splits - 1) / a.n_splits;
+    const int c_begin = blockIdx.z * per_split, c_end = min(n_chunks, c_begin + per_split);
+
+    // this wavefront's tile of 16 rows, this lane's row
+    const int r = blk_first + wave * 16 + lj;
+    const bool valid = r < rows;
+    const int i_tok = valid ? r / group_size : 0;
+    const int tok = qs + i_tok;
+    const int head = kh * group_size + (valid ? r % group_size : 0);
+    const int p_row = valid ? kv - n + i_tok : -1;
+    const int lo_row = (window > 0 && valid) ? max(0, p_row - window + 1) : 0;
+
+    // queries into LDS, zeros beyond the key size and in rows that belong to no token
+    {
+        const int pieces = krow / E;
+        for (int idx = tid; idx < ROWS * pieces; idx += THREADS) {
+            const int row = idx / pieces, c = idx % pieces;
+            const int rr = blk_first + row;
+            w_u32x4 v = w_u32x4{0u, 0u, 0u, 0u};
+            if (rr < rows && c * E < dk) {
+                const int t2 = qs + rr / group_size, h2 = kh * group_size + rr % group_size;
+                v = *reinterpret_cast<const w_u32x4*>(q + (static_cast<size_t>(t2) * nq + h2) * dk + c * E);
+            }
+            *reinterpret_cast<w_u32x4*>(q_s + row * krow + c * E) = v;
+        }
+    }
+
+    w_f32x4 o[DT];
+#pragma unroll
+    for (int d = 0; d < DT; ++d) o[d] = w_f32x4{0.f, 0.f, 0.f, 0.f};
+    float m_run = -INFINITY, l_run = 0.f;
+    const float scale = a.scale;
+    constexpr float kLog2e = 1.4426950408889634f;
+
+    for (int c = c_begin; c < c_end; ++c) {
+        const int tile = c < kept_chunks ? c : t_begin + (c - kept_chunks);
+        const int key0 = tile * KT;
+        __syncthreads();                  // the chunk before is read (and, the first time, the queries are written)
+        // ---- stage the chunk: keys [KT][dk], values transposed [dv][KT]; what no row of the workgroup sees is zeros
+        {
+            const int pieces = krow / E;
+            for (int idx = tid; idx < KT * pieces; idx += THREADS) {
+                const int key = idx / pieces, cc = idx % pieces;
+                const int j = key0 + key;
+                w_u32x4 v = w_u32x4{0u, 0u, 0u, 0u};
+                if (j <= p_max && (j >= lo_blk || j < keep) && cc * E < dk) {
+                    const long page = table[j / page_size];
+                    if (page >= 0)
+                        v = *reinterpret_cast<const w_u32x4*>(k_cache + ((page * nkv + kh) * page_size + j % page_size) * dk + cc * E);
+                }
+                *reinterpret_cast<w_u32x4*>(k_s + key * krow + cc * E) = v;
+            }
+            constexpr int VKP = KT / E;   // 16-byte pieces of a value row
+            for (int idx = tid; idx < DT * 16 * VKP; idx += THREADS) {
+                const int f = idx / VKP, v_key = (idx % VKP) * E;
+                const int j = key0 + v_key;
+                w_u32x4 v = w_u32x4{0u, 0u, 0u, 0u};
+                if (f < dv && j <= p_max && (j + E - 1 >= lo_blk || j < keep)) {
+                    const long page = table[j / page_size];
+                    if (page >= 0)
+                        v = *reinterpret_cast<const w_u32x4*>(v_cache + ((page * nkv + kh) * dv + f) * page_size + j % page_size);
+                    if (j + E > kv) {         // places of the page that no token has written yet may hold anything
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            if constexpr (sizeof(T) == 4) {
+                                if (j + e >= kv) v[e] = 0u;
+                            } else {
+                                if (j + 2 * e >= kv) v[e] = 0u;
+                                else if (j + 2 * e + 1 >= kv) v[e] &= 0x0000ffffu;
+                            }
+                        }
+                    }
+                }
+                if constexpr (sizeof(T) == 4) {
+                    *reinterpret_cast<w_u32x4*>(v_s + f * VROW + v_key) = v;
+                } else {
+                    // in the order in which a lane takes them: within 32 keys (quarter of the wavefront, tile, key)
+                    const int v_pos = (v_key / 32) * 32 + ((v_key % 16) / 4) * 8 + ((v_key % 32) / 16) * 4;
+                    *reinterpret_cast<w_u32x2*>(v_s + f * VROW + v_pos) = w_u32x2{v.x, v.y};
+                    *reinterpret_cast<w_u32x2*>(v_s + f * VROW + v_pos + 8) = w_u32x2{v.z, v.w};
+                }
+            }
+        }
+        __syncthreads();
+        // ---- scores of this wavefront's rows against the chunk's keys
+        w_f32x4 acc[NKT];
+        const T* ks = k_s + lj * krow + lg * E;
+        const T* qrow = q_s + (wave * 16 + lj) * krow + lg * E;
+#pragma unroll
+        for (int kt = 0; kt < NKT; ++kt) acc[kt] = w_f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int j = 0; j < n_pieces; ++j) {
+            const w_u32x4 qv = *reinterpret_cast<const w_u32x4*>(qrow + j * PF);
+#pragma unroll
+            for (int kt = 0; kt < NKT; ++kt) {
+                const w_u32x4 kvv = *reinterpret_cast<const w_u32x4*>(ks + kt * 16 * krow + j * PF);
+                acc[kt] = matrix_piece<T>(kvv, qv, acc[kt]);
+            }
+        }
+        matrix_results_ready();
+        // ---- mask, scale, one step of the online softmax (the lane's row; its four lanes share the statistics)
+        float mx = -INFINITY;
+#pragma unroll
+        for (int kt = 0; kt < NKT; ++kt)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const int key = key0 + kt * 16 + lg * 4 + v;
+                const bool seen = key <= p_row && (key >= lo_row || key < a.keep_first);
+                const float sc = seen ? acc[kt][v] * scale : -INFINITY;
+                acc[kt][v] = sc;
+                mx = fmaxf(mx, sc);
+            }
+        mx = fmaxf(mx, __shfl_xor(mx, 16, kWave));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
+        const float m_new = fmaxf(m_run, mx);
+        const float m_use = m_new == -INFINITY ? 0.f : m_new;      // a row that has seen nothing yet: every exp below is 0
+        const float alpha = __builtin_amdgcn_exp2f((m_run - m_use) * kLog2e);
+        l_run *= alpha;
+#pragma unroll
+        for (int d = 0; d < DT; ++d) {
+            o[d][0] *= alpha; o[d][1] *= alpha; o[d][2] *= alpha; o[d][3] *= alpha;
+        }
+        m_run = m_new;
+        float sum = 0.f;
+#pragma unroll
+        for (int kt = 0; kt < NKT; ++kt)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const float pv = __builtin_amdgcn_exp2f((acc[kt][v] - m_use) * kLog2e);
+                sum += pv;
+                acc[kt][v] = pv;
+            }
+        l_run += sum;
+        // ---- the probabilities as the second product's operand
+        w_u32x4 p[NP];
+        if constexpr (sizeof(T) == 2) {
+#pragma unroll
+            for (int j = 0; j < NP; ++j) {
+                w_bf16x8 pb;
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    pb[v] = static_cast<__bf16>(acc[2 * j][v]);
+                    pb[4 + v] = static_cast<__bf16>(acc[2 * j + 1][v]);
+                }
+                p[j] = __builtin_bit_cast(w_u32x4, pb);
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < NP; ++j) p[j] = __builtin_bit_cast(w_u32x4, acc[j]);
+        }
+        const T* vs = v_s + lj * VROW + lg * E;
+#pragma unroll
+        for (int d = 0; d < DT; ++d)
+#pragma unroll
+            for (int j = 0; j < NP; ++j) {
+                const w_u32x4 vv = *reinterpret_cast<const w_u32x4*>(vs + d * 16 * VROW + j * PF);
+                o[d] = matrix_piece<T>(vv, p[j], o[d]);
+            }
+    }
+    matrix_results_ready();
+    float l = l_run;
+    l += __shfl_xor(l, 16, kWave);
+    l += __shfl_xor(l, 32, kWave);
+    if (!valid) return;
+    if (a.n_splits > 1) {
+        const size_t row_at = (static_cast<size_t>(blockIdx.z) * a.n_tokens + tok) * nq + head;
+        float* po = a.part_o + row_at * dv + lg * 4;
+#pragma unroll
+        for (int d = 0; d < DT; ++d)
+            if (d * 16 < dv) *reinterpret_cast<float4*>(po + d * 16) = float4{o[d][0], o[d][1], o[d][2], o[d][3]};
+        if (lg == 0) {
+            a.part_ml[row_at * 2] = m_run;
+            a.part_ml[row_at * 2 + 1] = l;
+        }
+        return;
+    }
+    float weight = 1.0f;
+    if (a.sink != nullptr) {
+        const float sk = a.sink[head];
+        const float m_all = fmaxf(m_run, sk);
+        weight = __builtin_amdgcn_exp2f((m_run - m_all) * kLog2e);
+        l = l * weight + __builtin_amdgcn_exp2f((sk - m_all) * kLog2e);
+    }
+    const float inv = weight / l;
+    T* op = static_cast<T*>(a.out) + (static_cast<size_t>(tok) * nq + head) * dv + lg * 4;
+#pragma unroll
+    for (int d = 0; d < DT; ++d)
+        if (d * 16 < dv) store_four<T>(op + d * 16, o[d][0] * inv, o[d][1] * inv, o[d][2] * inv, o[d][3] * inv);
+}
+
+// The parts that the splits of a row's keys left, folded in the order of the splits, with the sink: one wavefront per
+// (token, head).
+template <typename T>
+__global__ __launch_bounds__(kWave) void window_attention_fold_kernel(const float* __restrict__ part_o,
+                                                                    const float* __restrict__ part_ml,
+                                                                    const float* __restrict__ sink, T* __restrict__ out,
+                                                                    int n_rows, int nq, int dv, int n_splits) {
+    const int row = blockIdx.x, lane = threadIdx.x;
+    float m_all = sink ? sink[row % nq] : -INFINITY;
+    for (int s = 0; s < n_splits; ++s) m_all = fmaxf(m_all, part_ml[(static_cast<size_t>(s) * n_rows + row) * 2]);
+    float l_all = sink ? expf(sink[row % nq] - m_all) : 0.f;
+    for (int s = 0; s < n_splits; ++s) {
+        const float* ml = part_ml + (static_cast<size_t>(s) * n_rows + row) * 2;
+        l_all = fmaf(ml[1], expf(ml[0] - m_all), l_all);
+    }
+    const float inv = 1.0f / l_all;
+    for (int d = lane; d < dv; d += kWave) {
+        float acc = 0.f;
+        for (int s = 0; s < n_splits; ++s) {
+            const size_t at = static_cast<size_t>(s) * n_rows + row;
+            acc = fmaf(part_o[at * dv + d], expf(part_ml[at * 2] - m_all), acc);
+        }
+        out[static_cast<size_t>(row) * dv + d] = from_float<T>(acc * inv);
+    }
+}
+
+template <typename T, int DT, int RT>
+static int launch_tiled(const WindowArgs& a, int max_rows, hipStream_t s) {
+    constexpr int E = 16 / sizeof(T), KT = sizeof(T) == 2 ? 64 : 32, PF = 4 * E;
+    const int krow = (a.dk + PF - 1) / PF * PF + E;
+    const size_t lds = (static_cast<size_t>(16 * RT + KT) * krow + static_cast<size_t>(DT) * 16 * (KT + E)) * sizeof(T);
+    if (lds > 160 * 1024) return EGPT_UNSUPPORTED_SIZE;
+    auto kernel = window_attention_tiled_kernel<T, DT, RT>;
+    if (lds > 48 * 1024) {
+        static bool raised = false;       // per instance of this template: the limit is asked for once
+        if (!raised) {
+            if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    160 * 1024) != hipSuccess)
+                return EGPT_LAUNCH_FAILED;
+            raised = true;
+        }
+    }
+    const int group_size = a.nq / a.nkv;
+    const int blocks = (max_rows * group_size + 16 * RT - 1) / (16 * RT) + a.n_seqs;
+    dim3 grid(blocks, a.nkv, a.n_splits);
+    kernel<<<grid, 64 * RT, lds, s>>>(a);
+    return EGPT_OK;
+}
+
+template <typename T, int RT>
+static int launch_tiled_for_dv(const WindowArgs& a, int max_rows, hipStream_t s) {
+    const int tiles = (a.dv + 15) / 16;
+    if (tiles <= 2) return launch_tiled<T, 2, RT>(a, max_rows, s);
+    if (tiles <= 4) return launch_tiled<T, 4, RT>(a, max_rows, s);
+    if (tiles <= 6) return launch_tiled<T, 6, RT>(a, max_rows, s);
+    if (tiles <= 8) return launch_tiled<T, 8, RT>(a, max_rows, s);
+    if (tiles <= 12) return launch_tiled<T, 12, RT>(a, max_rows, s);
+    if (tiles <= 16) return launch_tiled<T, 16, RT>(a, max_rows, s);
+    return EGPT_UNSUPPORTED_SIZE;
+}
+
 }  // namespace egpt
 
 using namespace egpt;
@@ -177,5 +543,46 @@ extern "C" int egpt_window_attention(const void* q, void* out, const void* k_cac
             static_cast<const bf16_t*>(v_cache), block_table, table_width, q_start, q_len, kv_len, n_seqs, nq, nkv, dk,
             dv, page_size, scale, window, keep_first, sink);
     EGPT_CHECK_LAUNCH();
+    return EGPT_OK;
+}
+
+extern "C" int egpt_window_attention_tiled(const void* q, void* out, float* part_o, float* part_ml, const void* k_cache,
+                                           const void* v_cache, const int32_t* block_table, int table_width,
+                                           const int32_t* q_start, const int32_t* q_len, const int32_t* kv_len, int n_seqs,
+                                           int n_tokens, int nq, int nkv, int dk, int dv, int page_size, float scale,
+                                           int window, int keep_first, const float* sink, int n_splits, int row_tiles,
+                                           int dtype, void* stream) {
+    if (!q || !out || !k_cache || !v_cache || !block_table || !q_start || !q_len || !kv_len) return EGPT_BAD_ARGUMENT;
+    if (n_seqs <= 0 || n_tokens < 0 || nq <= 0 || nkv <= 0 || nq % nkv != 0 || dk <= 0 || dv <= 0 || page_size <= 0 ||
+        table_width <= 0 || window < 0 || keep_first < 0 || n_splits < 1 || (dtype != 0 && dtype != 1) ||
+        (row_tiles != 1 && row_tiles != 4))
+        return EGPT_BAD_ARGUMENT;
+    if (n_splits > 1 && (!part_o || !part_ml)) return EGPT_BAD_ARGUMENT;
+    const int e = dtype == 0 ? 4 : 8;
+    if (dk % e || dv % 16 || dv > 256 || page_size % 16 || nkv > 65535 || n_splits > 65535) return EGPT_UNSUPPORTED_SIZE;
+    if (n_tokens == 0) return EGPT_OK;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    WindowArgs a;
+    a.q = q; a.out = out; a.part_o = part_o; a.part_ml = part_ml; a.k_cache = k_cache; a.v_cache = v_cache;
+    a.block_table = block_table; a.q_start = q_start; a.q_len = q_len; a.kv_len = kv_len; a.sink = sink;
+    a.table_width = table_width; a.n_seqs = n_seqs; a.n_tokens = n_tokens; a.nq = nq; a.nkv = nkv; a.dk = dk; a.dv = dv;
+    a.page_size = page_size; a.window = window; a.keep_first = keep_first; a.n_splits = n_splits; a.scale = scale;
+    int code;
+    if (dtype == 0)
+        code = row_tiles == 4 ? launch_tiled_for_dv<float, 4>(a, n_tokens, s) : launch_tiled_for_dv<float, 1>(a, n_tokens, s);
+    else
+        code = row_tiles == 4 ? launch_tiled_for_dv<bf16_t, 4>(a, n_tokens, s) : launch_tiled_for_dv<bf16_t, 1>(a, n_tokens, s);
+    if (code != EGPT_OK) return code;
+    EGPT_CHECK_LAUNCH();
+    if (n_splits > 1) {
+        if (dtype == 0)
+            window_attention_fold_kernel<float><<<n_tokens * nq, kWave, 0, s>>>(part_o, part_ml, sink, static_cast<float*>(out),
+                                                                               n_tokens * nq, nq, dv, n_splits);
+        else
+            window_attention_fold_kernel<bf16_t><<<n_tokens * nq, kWave, 0, s>>>(part_o, part_ml, sink,
+                                                                                static_cast<bf16_t*>(out), n_tokens * nq, nq,
+                                                                                dv, n_splits);
+        EGPT_CHECK_LAUNCH();
+    }
     return EGPT_OK;
 }

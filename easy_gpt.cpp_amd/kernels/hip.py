@@ -28,7 +28,7 @@ def _load_library() -> ctypes.CDLL:
         lib = ctypes.CDLL(path)
     except (build.BuildError, OSError) as e:
         raise KernelsUnavailable(f"the HIP kernel library could not be built or loaded: {e}") from e
-    if lib.egpt_abi_version() != 17:
+    if lib.egpt_abi_version() != 18:
         raise KernelsUnavailable(f"{path} has an unexpected ABI version")
     return lib
 
@@ -106,6 +106,8 @@ class HipKernels(KernelBackend):
             "egpt_latent_prep": [vp, i, i, vp, vp, vp, f, vp, f, i, vp, vp, vp, i, i, i, i, i, i, i, vp],
             "egpt_sigmoid_gate": [vp, i, vp, i, i, i, vp, i, i, i, vp],
             "egpt_window_attention": [vp, vp, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, i, f, i, i, vp, i, vp],
+            "egpt_window_attention_tiled": [vp, vp, vp, vp, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, i, f, i, i, vp, i, i,
+                                            i, vp],
         }
         lib.egpt_sample_workspace.restype = ctypes.c_size_t
         lib.egpt_sample_workspace.argtypes = [i, i]
@@ -945,9 +947,47 @@ class HipKernels(KernelBackend):
             raise ValueError(f"block table of width {width} cannot hold {max_kv_len} tokens at page size {page_size}")
         if dk > self.max_window_attention_dim or dv > self.max_window_attention_dim:
             raise ValueError(f"key size {dk} / value size {dv} is not supported (at most {self.max_window_attention_dim})")
+        shape = self._window_attention_shape(t, b, nq, nkv, dk, dv, page_size, window, keep_first, max_q_len, max_kv_len,
+                                             q.element_size())
+        if shape is not None:
+            row_tiles, n_splits = shape
+            part_o = part_ml = None
+            if n_splits > 1:
+                part_o = torch.empty((n_splits, t, nq, dv), dtype=_F32, device=q.device)
+                part_ml = torch.empty((n_splits, t, nq, 2), dtype=_F32, device=q.device)
+            self._run("egpt_window_attention_tiled", q.data_ptr(), out.data_ptr(), self._ptr(part_o), self._ptr(part_ml),
+                      k_cache.data_ptr(), v_cache.data_ptr(), block_table.data_ptr(), width, q_start.data_ptr(),
+                      q_len.data_ptr(), kv_len.data_ptr(), b, t, nq, nkv, dk, dv, page_size, float(scale), int(window),
+                      int(keep_first), self._ptr(sink), n_splits, row_tiles, dt, self._stream())
+            return
+        # sizes that the matrix-core kernel does not take: the general kernel
         self._run("egpt_window_attention", q.data_ptr(), out.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
                   block_table.data_ptr(), width, q_start.data_ptr(), q_len.data_ptr(), kv_len.data_ptr(), b, t, nq, nkv,
                   dk, dv, page_size, float(scale), int(window), int(keep_first), self._ptr(sink), dt, self._stream())
+
+    @staticmethod
+    def _window_attention_shape(t, b, nq, nkv, dk, dv, page_size, window, keep_first, max_q_len, max_kv_len, elem):
+        """(row tiles per workgroup, splits of the keys) of the matrix-core window attention, or None where its sizes
+        are not covered.  Prompt portions: workgroups of 64 rows that walk their keys alone.  Steps whose requests
+        bring so few rows that one tile of 16 holds them (single tokens): one wavefront per workgroup, and the chunks
+        of keys that a row sees dealt over enough workgroups to fill the GPU, a chunk or more each."""
+        e = 16 // elem
+        if dk % e or dv % 16 or dv > 256 or page_size % 16:
+            return None
+        chunk = 64 if elem == 2 else 32
+        group = nq // nkv
+        row_tiles = 4 if max_q_len * group > 16 else 1
+        krow = -(-dk // (4 * e)) * 4 * e + e
+        dv_tiles = next(n for n in (2, 4, 6, 8, 12, 16) if n * 16 >= dv)
+        if ((16 * row_tiles + chunk) * krow + dv_tiles * 16 * (chunk + e)) * elem > 160 * 1024:
+            return None
+        workgroups = (-(-t * group // (16 * row_tiles)) + b) * nkv
+        span = min(max_kv_len, window + chunk) if window else max_kv_len
+        chunks = -(-span // chunk) + (-(-min(keep_first, max_kv_len) // chunk) if window else 0)
+        n_splits = 1
+        if row_tiles == 1 and workgroups < 512:
+            n_splits = max(1, min(chunks, -(-512 // workgroups), 64))
+        return row_tiles, n_splits
 
     def swiglu(self, gate_up, out, row_ss=None, hidden=0, eps=0.0):
         """out = up * silu(gate) for gate_up act [T, 2I] or float32 partial sums [S, T, 2I].  row_ss float32
