@@ -220,15 +220,16 @@ struct WindowArgs {
     float scale;
 };
 
-template <typename T, int DT, int RT>
+template <typename T, int DT, int RT, int RW>
 __global__ __launch_bounds__(64 * RT) void window_attention_tiled_kernel(WindowArgs a) {
     constexpr int E = 16 / sizeof(T);             // elements in 16 bytes
     constexpr int KT = sizeof(T) == 2 ? 64 : 32;  // keys per chunk
     constexpr int NKT = KT / 16;                  // tiles of 16 keys in a chunk
     constexpr int PF = 4 * E;                     // features (or keys) that one matrix_piece sums over
     constexpr int NP = KT / PF;                   // pieces of a chunk's keys
-    constexpr int ROWS = 16 * RT, THREADS = 64 * RT;
+    constexpr int ROWS = 16 * RT * RW, THREADS = 64 * RT;     // a wavefront takes RW tiles of 16 rows
     constexpr int VROW = KT + E;                  // padded LDS row of values (elements)
+    constexpr int U = 8;                          // loads that a thread has in flight while a chunk is staged
     extern __shared__ __attribute__((aligned(16))) unsigned char window_smem[];
     const T* __restrict__ q = static_cast<const T*>(a.q);
     const T* __restrict__ k_cache = static_cast<const T*>(a.k_cache);
@@ -268,14 +269,19 @@ __global__ __launch_bounds__(64 * RT) void window_attention_tiled_kernel(WindowA
     const int per_split = (n_chunks + a.n_splits - 1) / a.n_splits;
     const int c_begin = blockIdx.z * per_split, c_end = min(n_chunks, c_begin + per_split);
 
-    // this wavefront's tile of 16 rows, this lane's row
-    const int r = blk_first + wave * 16 + lj;
-    const bool valid = r < rows;
-    const int i_tok = valid ? r / group_size : 0;
-    const int tok = qs + i_tok;
-    const int head = kh * group_size + (valid ? r % group_size : 0);
-    const int p_row = valid ? kv - n + i_tok : -1;
-    const int lo_row = (window > 0 && valid) ? max(0, p_row - window + 1) : 0;
+    // this wavefront's tiles of 16 rows, this lane's row in each
+    bool valid[RW];
+    int tok[RW], head[RW], p_row[RW], lo_row[RW];
+#pragma unroll
+    for (int w = 0; w < RW; ++w) {
+        const int r = blk_first + (wave * RW + w) * 16 + lj;
+        valid[w] = r < rows;
+        const int i_tok = valid[w] ? r / group_size : 0;
+        tok[w] = qs + i_tok;
+        head[w] = kh * group_size + (valid[w] ? r % group_size : 0);
+        p_row[w] = valid[w] ? kv - n + i_tok : -1;
+        lo_row[w] = (window > 0 && valid[w]) ? max(0, p_row[w] - window + 1) : 0;
+    }
 
     // queries into LDS, zeros beyond the key size and in rows that belong to no token
     {
@@ -292,10 +298,15 @@ __global__ __launch_bounds__(64 * RT) void window_attention_tiled_kernel(WindowA
         }
     }
 
-    w_f32x4 o[DT];
+    w_f32x4 o[RW][DT];
+    float m_run[RW], l_run[RW];
 #pragma unroll
-    for (int d = 0; d < DT; ++d) o[d] = w_f32x4{0.f, 0.f, 0.f, 0.f};
-    float m_run = -INFINITY, l_run = 0.f;
+    for (int w = 0; w < RW; ++w) {
+        m_run[w] = -INFINITY;
+        l_run[w] = 0.f;
+#pragma unroll
+        for (int d = 0; d < DT; ++d) o[w][d] = w_f32x4{0.f, 0.f, 0.f, 0.f};
+    }
     const float scale = a.scale;
     constexpr float kLog2e = 1.4426950408889634f;
 
@@ -303,116 +314,157 @@ __global__ __launch_bounds__(64 * RT) void window_attention_tiled_kernel(WindowA
         const int tile = c < kept_chunks ? c : t_begin + (c - kept_chunks);
         const int key0 = tile * KT;
         __syncthreads();                  // the chunk before is read (and, the first time, the queries are written)
-        // ---- stage the chunk: keys [KT][dk], values transposed [dv][KT]; what no row of the workgroup sees is zeros
+        // ---- stage the chunk: keys [KT][dk], values transposed [dv][KT]; what no row of the workgroup sees is zeros.
+        // U loads of a thread are issued before the first is stored.
         {
             const int pieces = krow / E;
-            for (int idx = tid; idx < KT * pieces; idx += THREADS) {
-                const int key = idx / pieces, cc = idx % pieces;
-                const int j = key0 + key;
-                w_u32x4 v = w_u32x4{0u, 0u, 0u, 0u};
-                if (j <= p_max && (j >= lo_blk || j < keep) && cc * E < dk) {
-                    const long page = table[j / page_size];
-                    if (page >= 0)
-                        v = *reinterpret_cast<const w_u32x4*>(k_cache + ((page * nkv + kh) * page_size + j % page_size) * dk + cc * E);
+            const int total = KT * pieces;
+            for (int base = tid; base < total; base += THREADS * U) {
+                w_u32x4 regs[U];
+                long pages[U];
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    const int idx = base + u * THREADS;
+                    const int j = key0 + idx / pieces, cc = idx % pieces;
+                    pages[u] = -1;
+                    if (idx < total && j <= p_max && (j >= lo_blk || j < keep) && cc * E < dk) pages[u] = table[j / page_size];
                 }
-                *reinterpret_cast<w_u32x4*>(k_s + key * krow + cc * E) = v;
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    const int idx = base + u * THREADS;
+                    const int j = key0 + idx / pieces, cc = idx % pieces;
+                    regs[u] = w_u32x4{0u, 0u, 0u, 0u};
+                    if (pages[u] >= 0)
+                        regs[u] = *reinterpret_cast<const w_u32x4*>(k_cache + ((pages[u] * nkv + kh) * page_size + j % page_size) * dk + cc * E);
+                }
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    const int idx = base + u * THREADS;
+                    if (idx < total) *reinterpret_cast<w_u32x4*>(k_s + (idx / pieces) * krow + (idx % pieces) * E) = regs[u];
+                }
             }
             constexpr int VKP = KT / E;   // 16-byte pieces of a value row
-            for (int idx = tid; idx < DT * 16 * VKP; idx += THREADS) {
-                const int f = idx / VKP, v_key = (idx % VKP) * E;
-                const int j = key0 + v_key;
-                w_u32x4 v = w_u32x4{0u, 0u, 0u, 0u};
-                if (f < dv && j <= p_max && (j + E - 1 >= lo_blk || j < keep)) {
-                    const long page = table[j / page_size];
-                    if (page >= 0)
-                        v = *reinterpret_cast<const w_u32x4*>(v_cache + ((page * nkv + kh) * dv + f) * page_size + j % page_size);
-                    if (j + E > kv) {         // places of the page that no token has written yet may hold anything
+            constexpr int VTOTAL = DT * 16 * VKP;
+            for (int base = tid; base < VTOTAL; base += THREADS * U) {
+                w_u32x4 regs[U];
+                long pages[U];
 #pragma unroll
-                        for (int e = 0; e < 4; ++e) {
-                            if constexpr (sizeof(T) == 4) {
-                                if (j + e >= kv) v[e] = 0u;
-                            } else {
-                                if (j + 2 * e >= kv) v[e] = 0u;
-                                else if (j + 2 * e + 1 >= kv) v[e] &= 0x0000ffffu;
+                for (int u = 0; u < U; ++u) {
+                    const int idx = base + u * THREADS;
+                    const int f = idx / VKP, j = key0 + (idx % VKP) * E;
+                    pages[u] = -1;
+                    if (idx < VTOTAL && f < dv && j <= p_max && (j + E - 1 >= lo_blk || j < keep)) pages[u] = table[j / page_size];
+                }
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    const int idx = base + u * THREADS;
+                    const int f = idx / VKP, j = key0 + (idx % VKP) * E;
+                    w_u32x4 v = w_u32x4{0u, 0u, 0u, 0u};
+                    if (pages[u] >= 0) {
+                        v = *reinterpret_cast<const w_u32x4*>(v_cache + ((pages[u] * nkv + kh) * dv + f) * page_size + j % page_size);
+                        if (j + E > kv) {         // places of the page that no token has written yet may hold anything
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) {
+                                if constexpr (sizeof(T) == 4) {
+                                    if (j + e >= kv) v[e] = 0u;
+                                } else {
+                                    if (j + 2 * e >= kv) v[e] = 0u;
+                                    else if (j + 2 * e + 1 >= kv) v[e] &= 0x0000ffffu;
+                                }
                             }
                         }
                     }
+                    regs[u] = v;
                 }
-                if constexpr (sizeof(T) == 4) {
-                    *reinterpret_cast<w_u32x4*>(v_s + f * VROW + v_key) = v;
-                } else {
-                    // in the order in which a lane takes them: within 32 keys (quarter of the wavefront, tile, key)
-                    const int v_pos = (v_key / 32) * 32 + ((v_key % 16) / 4) * 8 + ((v_key % 32) / 16) * 4;
-                    *reinterpret_cast<w_u32x2*>(v_s + f * VROW + v_pos) = w_u32x2{v.x, v.y};
-                    *reinterpret_cast<w_u32x2*>(v_s + f * VROW + v_pos + 8) = w_u32x2{v.z, v.w};
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    const int idx = base + u * THREADS;
+                    if (idx >= VTOTAL) continue;
+                    const int f = idx / VKP, v_key = (idx % VKP) * E;
+                    if constexpr (sizeof(T) == 4) {
+                        *reinterpret_cast<w_u32x4*>(v_s + f * VROW + v_key) = regs[u];
+                    } else {
+                        // in the order in which a lane takes them: within 32 keys (quarter of the wavefront, tile, key)
+                        const int v_pos = (v_key / 32) * 32 + ((v_key % 16) / 4) * 8 + ((v_key % 32) / 16) * 4;
+                        *reinterpret_cast<w_u32x2*>(v_s + f * VROW + v_pos) = w_u32x2{regs[u].x, regs[u].y};
+                        *reinterpret_cast<w_u32x2*>(v_s + f * VROW + v_pos + 8) = w_u32x2{regs[u].z, regs[u].w};
+                    }
                 }
             }
         }
         __syncthreads();
-        // ---- scores of this wavefront's rows against the chunk's keys
-        w_f32x4 acc[NKT];
+        // ---- scores of this wavefront's rows against the chunk's keys: a key operand serves all of its row tiles
+        w_f32x4 acc[RW][NKT];
         const T* ks = k_s + lj * krow + lg * E;
-        const T* qrow = q_s + (wave * 16 + lj) * krow + lg * E;
+        const T* qrow = q_s + (wave * RW * 16 + lj) * krow + lg * E;
 #pragma unroll
-        for (int kt = 0; kt < NKT; ++kt) acc[kt] = w_f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int w = 0; w < RW; ++w)
+#pragma unroll
+            for (int kt = 0; kt < NKT; ++kt) acc[w][kt] = w_f32x4{0.f, 0.f, 0.f, 0.f};
         for (int j = 0; j < n_pieces; ++j) {
-            const w_u32x4 qv = *reinterpret_cast<const w_u32x4*>(qrow + j * PF);
+            w_u32x4 qv[RW];
+#pragma unroll
+            for (int w = 0; w < RW; ++w) qv[w] = *reinterpret_cast<const w_u32x4*>(qrow + w * 16 * krow + j * PF);
 #pragma unroll
             for (int kt = 0; kt < NKT; ++kt) {
                 const w_u32x4 kvv = *reinterpret_cast<const w_u32x4*>(ks + kt * 16 * krow + j * PF);
-                acc[kt] = matrix_piece<T>(kvv, qv, acc[kt]);
+#pragma unroll
+                for (int w = 0; w < RW; ++w) acc[w][kt] = matrix_piece<T>(kvv, qv[w], acc[w][kt]);
             }
         }
         matrix_results_ready();
-        // ---- mask, scale, one step of the online softmax (the lane's row; its four lanes share the statistics)
-        float mx = -INFINITY;
+        // ---- mask, scale, one step of the online softmax (the lane's rows; a row's four lanes share the statistics)
+        w_u32x4 p[RW][NP];
 #pragma unroll
-        for (int kt = 0; kt < NKT; ++kt)
+        for (int w = 0; w < RW; ++w) {
+            float mx = -INFINITY;
 #pragma unroll
-            for (int v = 0; v < 4; ++v) {
-                const int key = key0 + kt * 16 + lg * 4 + v;
-                const bool seen = key <= p_row && (key >= lo_row || key < a.keep_first);
-                const float sc = seen ? acc[kt][v] * scale : -INFINITY;
-                acc[kt][v] = sc;
-                mx = fmaxf(mx, sc);
-            }
-        mx = fmaxf(mx, __shfl_xor(mx, 16, kWave));
-        mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
-        const float m_new = fmaxf(m_run, mx);
-        const float m_use = m_new == -INFINITY ? 0.f : m_new;      // a row that has seen nothing yet: every exp below is 0
-        const float alpha = __builtin_amdgcn_exp2f((m_run - m_use) * kLog2e);
-        l_run *= alpha;
-#pragma unroll
-        for (int d = 0; d < DT; ++d) {
-            o[d][0] *= alpha; o[d][1] *= alpha; o[d][2] *= alpha; o[d][3] *= alpha;
-        }
-        m_run = m_new;
-        float sum = 0.f;
-#pragma unroll
-        for (int kt = 0; kt < NKT; ++kt)
-#pragma unroll
-            for (int v = 0; v < 4; ++v) {
-                const float pv = __builtin_amdgcn_exp2f((acc[kt][v] - m_use) * kLog2e);
-                sum += pv;
-                acc[kt][v] = pv;
-            }
-        l_run += sum;
-        // ---- the probabilities as the second product's operand
-        w_u32x4 p[NP];
-        if constexpr (sizeof(T) == 2) {
-#pragma unroll
-            for (int j = 0; j < NP; ++j) {
-                w_bf16x8 pb;
+            for (int kt = 0; kt < NKT; ++kt)
 #pragma unroll
                 for (int v = 0; v < 4; ++v) {
-                    pb[v] = static_cast<__bf16>(acc[2 * j][v]);
-                    pb[4 + v] = static_cast<__bf16>(acc[2 * j + 1][v]);
+                    const int key = key0 + kt * 16 + lg * 4 + v;
+                    const bool seen = key <= p_row[w] && (key >= lo_row[w] || key < a.keep_first);
+                    const float sc = seen ? acc[w][kt][v] * scale : -INFINITY;
+                    acc[w][kt][v] = sc;
+                    mx = fmaxf(mx, sc);
                 }
-                p[j] = __builtin_bit_cast(w_u32x4, pb);
-            }
-        } else {
+            mx = fmaxf(mx, __shfl_xor(mx, 16, kWave));
+            mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
+            const float m_new = fmaxf(m_run[w], mx);
+            const float m_use = m_new == -INFINITY ? 0.f : m_new;      // a row that has seen nothing yet: every exp below is 0
+            const float alpha = __builtin_amdgcn_exp2f((m_run[w] - m_use) * kLog2e);
+            l_run[w] *= alpha;
 #pragma unroll
-            for (int j = 0; j < NP; ++j) p[j] = __builtin_bit_cast(w_u32x4, acc[j]);
+            for (int d = 0; d < DT; ++d) {
+                o[w][d][0] *= alpha; o[w][d][1] *= alpha; o[w][d][2] *= alpha; o[w][d][3] *= alpha;
+            }
+            m_run[w] = m_new;
+            float sum = 0.f;
+#pragma unroll
+            for (int kt = 0; kt < NKT; ++kt)
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    const float pv = __builtin_amdgcn_exp2f((acc[w][kt][v] - m_use) * kLog2e);
+                    sum += pv;
+                    acc[w][kt][v] = pv;
+                }
+            l_run[w] += sum;
+            // the probabilities as the second product's operand
+            if constexpr (sizeof(T) == 2) {
+#pragma unroll
+                for (int j = 0; j < NP; ++j) {
+                    w_bf16x8 pb;
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) {
+                        pb[v] = static_cast<__bf16>(acc[w][2 * j][v]);
+                        pb[4 + v] = static_cast<__bf16>(acc[w][2 * j + 1][v]);
+                    }
+                    p[w][j] = __builtin_bit_cast(w_u32x4, pb);
+                }
+            } else {
+#pragma unroll
+                for (int j = 0; j < NP; ++j) p[w][j] = __builtin_bit_cast(w_u32x4, acc[w][j]);
+            }
         }
         const T* vs = v_s + lj * VROW + lg * E;
 #pragma unroll
@@ -420,38 +472,43 @@ __global__ __launch_bounds__(64 * RT) void window_attention_tiled_kernel(WindowA
 #pragma unroll
             for (int j = 0; j < NP; ++j) {
                 const w_u32x4 vv = *reinterpret_cast<const w_u32x4*>(vs + d * 16 * VROW + j * PF);
-                o[d] = matrix_piece<T>(vv, p[j], o[d]);
+#pragma unroll
+                for (int w = 0; w < RW; ++w) o[w][d] = matrix_piece<T>(vv, p[w][j], o[w][d]);
             }
     }
     matrix_results_ready();
-    float l = l_run;
-    l += __shfl_xor(l, 16, kWave);
-    l += __shfl_xor(l, 32, kWave);
-    if (!valid) return;
-    if (a.n_splits > 1) {
-        const size_t row_at = (static_cast<size_t>(blockIdx.z) * a.n_tokens + tok) * nq + head;
-        float* po = a.part_o + row_at * dv + lg * 4;
+#pragma unroll
+    for (int w = 0; w < RW; ++w) {
+        float l = l_run[w];
+        l += __shfl_xor(l, 16, kWave);
+        l += __shfl_xor(l, 32, kWave);
+        if (!valid[w]) continue;
+        if (a.n_splits > 1) {
+            const size_t row_at = (static_cast<size_t>(blockIdx.z) * a.n_tokens + tok[w]) * nq + head[w];
+            float* po = a.part_o + row_at * dv + lg * 4;
+#pragma unroll
+            for (int d = 0; d < DT; ++d)
+                if (d * 16 < dv) *reinterpret_cast<float4*>(po + d * 16) = float4{o[w][d][0], o[w][d][1], o[w][d][2], o[w][d][3]};
+            if (lg == 0) {
+                a.part_ml[row_at * 2] = m_run[w];
+                a.part_ml[row_at * 2 + 1] = l;
+            }
+            continue;
+        }
+        float weight = 1.0f;
+        if (a.sink != nullptr) {
+            const float sk = a.sink[head[w]];
+            const float m_all = fmaxf(m_run[w], sk);
+            weight = __builtin_amdgcn_exp2f((m_run[w] - m_all) * kLog2e);
+            l = l * weight + __builtin_amdgcn_exp2f((sk - m_all) * kLog2e);
+        }
+        const float inv = weight / l;
+        T* op = static_cast<T*>(a.out) + (static_cast<size_t>(tok[w]) * nq + head[w]) * dv + lg * 4;
 #pragma unroll
         for (int d = 0; d < DT; ++d)
-            if (d * 16 < dv) *reinterpret_cast<float4*>(po + d * 16) = float4{o[d][0], o[d][1], o[d][2], o[d][3]};
-        if (lg == 0) {
-            a.part_ml[row_at * 2] = m_run;
-            a.part_ml[row_at * 2 + 1] = l;
-        }
-        return;
+            if (d * 16 < dv)
+                store_four<T>(op + d * 16, o[w][d][0] * inv, o[w][d][1] * inv, o[w][d][2] * inv, o[w][d][3] * inv);
     }
-    float weight = 1.0f;
-    if (a.sink != nullptr) {
-        const float sk = a.sink[head];
-        const float m_all = fmaxf(m_run, sk);
-        weight = __builtin_amdgcn_exp2f((m_run - m_all) * kLog2e);
-        l = l * weight + __builtin_amdgcn_exp2f((sk - m_all) * kLog2e);
-    }
-    const float inv = weight / l;
-    T* op = static_cast<T*>(a.out) + (static_cast<size_t>(tok) * nq + head) * dv + lg * 4;
-#pragma unroll
-    for (int d = 0; d < DT; ++d)
-        if (d * 16 < dv) store_four<T>(op + d * 16, o[d][0] * inv, o[d][1] * inv, o[d][2] * inv, o[d][3] * inv);
 }
 
 // The parts that the splits of a row's keys left, folded in the order of the splits, with the sink: one wavefront per
@@ -461,32 +518,37 @@ __global__ __launch_bounds__(kWave) void window_attention_fold_kernel(const floa
                                                                     const float* __restrict__ part_ml,
                                                                     const float* __restrict__ sink, T* __restrict__ out,
                                                                     int n_rows, int nq, int dv, int n_splits) {
+    __shared__ float weights[kWave];           // at most 64 splits
     const int row = blockIdx.x, lane = threadIdx.x;
-    float m_all = sink ? sink[row % nq] : -INFINITY;
-    for (int s = 0; s < n_splits; ++s) m_all = fmaxf(m_all, part_ml[(static_cast<size_t>(s) * n_rows + row) * 2]);
-    float l_all = sink ? expf(sink[row % nq] - m_all) : 0.f;
-    for (int s = 0; s < n_splits; ++s) {
-        const float* ml = part_ml + (static_cast<size_t>(s) * n_rows + row) * 2;
-        l_all = fmaf(ml[1], expf(ml[0] - m_all), l_all);
+    float m = -INFINITY, l = 0.f;
+    if (lane < n_splits) {
+        const float* ml = part_ml + (static_cast<size_t>(lane) * n_rows + row) * 2;
+        m = ml[0];
+        l = ml[1];
     }
+    float m_all = wave_max(m);
+    if (sink) m_all = fmaxf(m_all, sink[row % nq]);
+    const float w = lane < n_splits ? expf(m - m_all) : 0.f;     // exp(-inf) = 0 for a split that saw nothing
+    float l_all = wave_sum(l * w);
+    if (sink) l_all += expf(sink[row % nq] - m_all);
+    weights[lane] = w;
+    __syncthreads();
     const float inv = 1.0f / l_all;
     for (int d = lane; d < dv; d += kWave) {
         float acc = 0.f;
-        for (int s = 0; s < n_splits; ++s) {
-            const size_t at = static_cast<size_t>(s) * n_rows + row;
-            acc = fmaf(part_o[at * dv + d], expf(part_ml[at * 2] - m_all), acc);
-        }
+        for (int s = 0; s < n_splits; ++s)
+            acc = fmaf(part_o[(static_cast<size_t>(s) * n_rows + row) * dv + d], weights[s], acc);
         out[static_cast<size_t>(row) * dv + d] = from_float<T>(acc * inv);
     }
 }
 
-template <typename T, int DT, int RT>
+template <typename T, int DT, int RT, int RW>
 static int launch_tiled(const WindowArgs& a, int max_rows, hipStream_t s) {
-    constexpr int E = 16 / sizeof(T), KT = sizeof(T) == 2 ? 64 : 32, PF = 4 * E;
+    constexpr int E = 16 / sizeof(T), KT = sizeof(T) == 2 ? 64 : 32, PF = 4 * E, ROWS = 16 * RT * RW;
     const int krow = (a.dk + PF - 1) / PF * PF + E;
-    const size_t lds = (static_cast<size_t>(16 * RT + KT) * krow + static_cast<size_t>(DT) * 16 * (KT + E)) * sizeof(T);
+    const size_t lds = (static_cast<size_t>(ROWS + KT) * krow + static_cast<size_t>(DT) * 16 * (KT + E)) * sizeof(T);
     if (lds > 160 * 1024) return EGPT_UNSUPPORTED_SIZE;
-    auto kernel = window_attention_tiled_kernel<T, DT, RT>;
+    auto kernel = window_attention_tiled_kernel<T, DT, RT, RW>;
     if (lds > 48 * 1024) {
         static bool raised = false;       // per instance of this template: the limit is asked for once
         if (!raised) {
@@ -497,21 +559,29 @@ static int launch_tiled(const WindowArgs& a, int max_rows, hipStream_t s) {
         }
     }
     const int group_size = a.nq / a.nkv;
-    const int blocks = (max_rows * group_size + 16 * RT - 1) / (16 * RT) + a.n_seqs;
+    const int blocks = (max_rows * group_size + ROWS - 1) / ROWS + a.n_seqs;
     dim3 grid(blocks, a.nkv, a.n_splits);
     kernel<<<grid, 64 * RT, lds, s>>>(a);
     return EGPT_OK;
 }
 
-template <typename T, int RT>
-static int launch_tiled_for_dv(const WindowArgs& a, int max_rows, hipStream_t s) {
+// row_tiles: 1 (a wavefront with 16 rows), 4 (four wavefronts with 16 rows each) or 8 (four with 32 rows each)
+template <typename T, int DT>
+static int launch_tiled_for_rows(const WindowArgs& a, int max_rows, int row_tiles, hipStream_t s) {
+    if (row_tiles == 8) return launch_tiled<T, DT, 4, 2>(a, max_rows, s);
+    if (row_tiles == 4) return launch_tiled<T, DT, 4, 1>(a, max_rows, s);
+    return launch_tiled<T, DT, 1, 1>(a, max_rows, s);
+}
+
+template <typename T>
+static int launch_tiled_for_dv(const WindowArgs& a, int max_rows, int row_tiles, hipStream_t s) {
     const int tiles = (a.dv + 15) / 16;
-    if (tiles <= 2) return launch_tiled<T, 2, RT>(a, max_rows, s);
-    if (tiles <= 4) return launch_tiled<T, 4, RT>(a, max_rows, s);
-    if (tiles <= 6) return launch_tiled<T, 6, RT>(a, max_rows, s);
-    if (tiles <= 8) return launch_tiled<T, 8, RT>(a, max_rows, s);
-    if (tiles <= 12) return launch_tiled<T, 12, RT>(a, max_rows, s);
-    if (tiles <= 16) return launch_tiled<T, 16, RT>(a, max_rows, s);
+    if (tiles <= 2) return launch_tiled_for_rows<T, 2>(a, max_rows, row_tiles, s);
+    if (tiles <= 4) return launch_tiled_for_rows<T, 4>(a, max_rows, row_tiles, s);
+    if (tiles <= 6) return launch_tiled_for_rows<T, 6>(a, max_rows, row_tiles, s);
+    if (tiles <= 8) return launch_tiled_for_rows<T, 8>(a, max_rows, row_tiles, s);
+    if (tiles <= 12) return launch_tiled_for_rows<T, 12>(a, max_rows, row_tiles, s);
+    if (tiles <= 16) return launch_tiled_for_rows<T, 16>(a, max_rows, row_tiles, s);
     return EGPT_UNSUPPORTED_SIZE;
 }
 
@@ -555,11 +625,11 @@ extern "C" int egpt_window_attention_tiled(const void* q, void* out, float* part
     if (!q || !out || !k_cache || !v_cache || !block_table || !q_start || !q_len || !kv_len) return EGPT_BAD_ARGUMENT;
     if (n_seqs <= 0 || n_tokens < 0 || nq <= 0 || nkv <= 0 || nq % nkv != 0 || dk <= 0 || dv <= 0 || page_size <= 0 ||
         table_width <= 0 || window < 0 || keep_first < 0 || n_splits < 1 || (dtype != 0 && dtype != 1) ||
-        (row_tiles != 1 && row_tiles != 4))
+        (row_tiles != 1 && row_tiles != 4 && row_tiles != 8))
         return EGPT_BAD_ARGUMENT;
     if (n_splits > 1 && (!part_o || !part_ml)) return EGPT_BAD_ARGUMENT;
     const int e = dtype == 0 ? 4 : 8;
-    if (dk % e || dv % 16 || dv > 256 || page_size % 16 || nkv > 65535 || n_splits > 65535) return EGPT_UNSUPPORTED_SIZE;
+    if (dk % e || dv % 16 || dv > 256 || page_size % 16 || nkv > 65535 || n_splits > 64) return EGPT_UNSUPPORTED_SIZE;
     if (n_tokens == 0) return EGPT_OK;
     hipStream_t s = static_cast<hipStream_t>(stream);
     WindowArgs a;
@@ -569,9 +639,9 @@ extern "C" int egpt_window_attention_tiled(const void* q, void* out, float* part
     a.page_size = page_size; a.window = window; a.keep_first = keep_first; a.n_splits = n_splits; a.scale = scale;
     int code;
     if (dtype == 0)
-        code = row_tiles == 4 ? launch_tiled_for_dv<float, 4>(a, n_tokens, s) : launch_tiled_for_dv<float, 1>(a, n_tokens, s);
+        code = launch_tiled_for_dv<float>(a, n_tokens, row_tiles, s);
     else
-        code = row_tiles == 4 ? launch_tiled_for_dv<bf16_t, 4>(a, n_tokens, s) : launch_tiled_for_dv<bf16_t, 1>(a, n_tokens, s);
+        code = launch_tiled_for_dv<bf16_t>(a, n_tokens, row_tiles, s);
     if (code != EGPT_OK) return code;
     EGPT_CHECK_LAUNCH();
     if (n_splits > 1) {

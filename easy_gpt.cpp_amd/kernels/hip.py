@@ -965,6 +965,8 @@ class HipKernels(KernelBackend):
                   block_table.data_ptr(), width, q_start.data_ptr(), q_len.data_ptr(), kv_len.data_ptr(), b, t, nq, nkv,
                   dk, dv, page_size, float(scale), int(window), int(keep_first), self._ptr(sink), dt, self._stream())
 
+    wide_rows_from = 16384          # rows of a step from which the window attention gives a wavefront 32 of them
+
     @staticmethod
     def _window_attention_shape(t, b, nq, nkv, dk, dv, page_size, window, keep_first, max_q_len, max_kv_len, elem):
         """(row tiles per workgroup, splits of the keys) of the matrix-core window attention, or None where its sizes
@@ -976,10 +978,14 @@ class HipKernels(KernelBackend):
             return None
         chunk = 64 if elem == 2 else 32
         group = nq // nkv
-        row_tiles = 4 if max_q_len * group > 16 else 1
+        # many rows: 32 to a wavefront, which halves the reads of a chunk's keys and values from LDS per row
+        row_tiles = 1 if max_q_len * group <= 16 else 4 if t * group * nkv < HipKernels.wide_rows_from else 8
         krow = -(-dk // (4 * e)) * 4 * e + e
         dv_tiles = next(n for n in (2, 4, 6, 8, 12, 16) if n * 16 >= dv)
-        if ((16 * row_tiles + chunk) * krow + dv_tiles * 16 * (chunk + e)) * elem > 160 * 1024:
+        lds = lambda tiles: ((16 * tiles + chunk) * krow + dv_tiles * 16 * (chunk + e)) * elem
+        if row_tiles == 8 and lds(8) > 160 * 1024:
+            row_tiles = 4
+        if lds(row_tiles) > 160 * 1024:
             return None
         workgroups = (-(-t * group // (16 * row_tiles)) + b) * nkv
         span = min(max_kv_len, window + chunk) if window else max_kv_len

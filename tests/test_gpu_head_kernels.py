@@ -206,6 +206,32 @@ def test_attention_against_plain(k, dtype, nq, nkv, dk, dv, window, keep_first, 
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("nq, nkv, dk, dv", [(4, 2, 16, 32), (8, 1, 128, 96), (6, 2, 72, 16)])
+@pytest.mark.parametrize("window, keep_first, with_sink", [(0, 0, True), (70, 0, False), (40, 33, True)])
+def test_attention_with_32_rows_to_a_wavefront(k, dtype, nq, nkv, dk, dv, window, keep_first, with_sink):
+    """The shape that steps of thousands of rows take, forced on a small one."""
+    from easy_gpt.cpp_amd.kernels.hip import HipKernels
+
+    n, ps = 333, 16
+    keys, values = rnd(n, nkv, dk, seed=81).to(dtype), rnd(n, nkv, dv, seed=82).to(dtype)
+    q = rnd(n, nq, dk, seed=83, scale=1.5).to(dtype)
+    sink = rnd(nq, seed=84, scale=2.0) if with_sink else None
+    scale = 1.7 / math.sqrt(dk)
+    k_cache, v_cache, table = paged(keys, values, ps, dtype, seed=85)
+    want = plain_attention(q, keys, values, 0, scale, window, keep_first, sink)
+    before = HipKernels.wide_rows_from
+    HipKernels.wide_rows_from = 0
+    try:
+        assert HipKernels._window_attention_shape(n, 1, nq, nkv, dk, dv, ps, window, keep_first, n, n, q.element_size())[0] == 8
+        got = run_attention(k, q, k_cache, v_cache, table, n, ps, scale, window, keep_first, sink, dv)
+        close(got, want, dtype, "whole prompt")
+        got = run_attention(k, q[200:301], k_cache, v_cache, table, 301, ps, scale, window, keep_first, sink, dv)
+        close(got, want[200:301], dtype, "a portion")
+    finally:
+        HipKernels.wide_rows_from = before
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_one_far_key_among_hundreds_is_found(k, dtype):
     """Key 3 of 900 fits the query; every other key is noise.  The output is key 3's value."""
     n, ps, dk, dv = 900, 16, 64, 32
