@@ -153,9 +153,9 @@ int egpt_window_attention(const void* q, void* out, const void* k_cache, const v
                           int table_width, const int32_t* q_start, const int32_t* q_len, const int32_t* kv_len,
                           int n_seqs, int n_tokens, int nq, int nkv, int dk, int dv, int page_size, float scale,
                           int window, int keep_first, const float* sink, int dtype, void* stream);
-// The same on the matrix cores: dk a multiple of 4 (float32) or 8 (bfloat16), dv a multiple of 16 up to 256, page_size a
-// multiple of 16.  row_tiles: tiles of 16 rows to a workgroup: 8 (four wavefronts with 32 rows each) or 4 (with 16 each)
-// for prompt portions, 1 (one wavefront) for single tokens.  With
+// The same on the matrix cores: dk a multiple of 4 (float32) or 8 (bfloat16) up to 256, dv a multiple of 16 up to 256,
+// page_size a multiple of 16.  row_tiles: tiles of 16 rows to a workgroup of four wavefronts: 8 (32 rows to a wavefront)
+// or 4 (16).  With
 // n_splits > 1 the chunks of keys of a workgroup's rows are dealt over as many workgroups, whose results part_o
 // [n_splits][n_tokens][nq][dv] and part_ml [n_splits][n_tokens][nq][2] (float32) a second kernel folds.
 int egpt_window_attention_tiled(const void* q, void* out, float* part_o, float* part_ml, const void* k_cache,

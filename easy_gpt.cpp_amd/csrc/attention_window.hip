@@ -151,17 +151,19 @@ __global__ __launch_bounds__(64 * kSimpleWaves) void window_attention_simple_ker
 
 
 // ---------------------------------------------------------------------------------------------- on the matrix cores
-// The same attention for key sizes that are multiples of 16 bytes' worth of elements, value sizes that are multiples
-// of 16 up to 256, and page sizes that are multiples of 16.  Rows are (token, query head) pairs of one key/value
+// The same attention for key sizes up to 256 that are multiples of 16 bytes' worth of elements, value sizes that are
+// multiples of 16 up to 256, and page sizes that are multiples of 16.  Rows are (token, query head) pairs of one key/value
 // head's group, 16 to a wavefront; the scores are computed transposed, S^T[key, row] = K[key, :] . Q[row, :], so that a
 // lane holds scores of one row, the row's statistics are per-lane scalars and the probabilities are the second
 // product's operand as they lie in registers: O^T[feature, row] += V^T[feature, key] . P^T[key, row].
 //   bfloat16: v_mfma_f32_16x16x32_bf16, a lane's 16 bytes of an operand are 8 features (or 8 keys);
 //   float32:  v_mfma_f32_16x16x4_f32 (float32 operands and accumulation), a lane's 16 bytes are 4 features (or 4 keys).
-// A workgroup of RT wavefronts takes 16 * RT rows of one request and key/value head and walks the chunks of KT keys
+// A workgroup of RT wavefronts takes 16 * RW * RT rows of one request and key/value head (RW tiles of 16 rows to a
+// wavefront, which then uses every key and value operand it reads from LDS RW times) and walks the chunks of KT keys
 // that any of its rows can see: those that hold kept first tokens, then those of the window.  A chunk's keys and values
-// are staged through LDS and shared by the wavefronts; the queries lie in LDS too, so the key size is a run-time
-// number (the value size, which sizes the accumulators, is a template parameter in steps).  With n_splits > 1 the
+// are staged through LDS and shared by the wavefronts, the next chunk's loads in flight meanwhile; the queries lie in
+// LDS too, so the key size is a run-time number (the value size, which sizes the accumulators, is a template
+// parameter in steps).  With n_splits > 1 the
 // chunks of a workgroup's rows are dealt over as many workgroups (grid z), which leave unnormalised results
 // part_o [split][token][head][dv] and (maximum, sum) part_ml [split][token][head][2] that window_attention_fold_kernel
 // combines; that kernel also adds the sink.  With one split the kernel finishes the rows itself.
@@ -229,7 +231,9 @@ __global__ __launch_bounds__(64 * RT) void window_attention_tiled_kernel(WindowA
     constexpr int NP = KT / PF;                   // pieces of a chunk's keys
     constexpr int ROWS = 16 * RT * RW, THREADS = 64 * RT;     // a wavefront takes RW tiles of 16 rows
     constexpr int VROW = KT + E;                  // padded LDS row of values (elements)
-    constexpr int U = 8;                          // loads that a thread has in flight while a chunk is staged
+    constexpr int U = 8;                          // loads that a thread has in flight while the queries are staged
+    constexpr int KU = 8;                         // 16-byte pieces of a chunk's keys per thread: 64 keys of 256 features
+    constexpr int VU = (DT * 16 * (KT / E) + THREADS - 1) / THREADS;      // and of its values
     extern __shared__ __attribute__((aligned(16))) unsigned char window_smem[];
     const T* __restrict__ q = static_cast<const T*>(a.q);
     const T* __restrict__ k_cache = static_cast<const T*>(a.k_cache);
@@ -237,6 +241,7 @@ __global__ __launch_bounds__(64 * RT) void window_attention_tiled_kernel(WindowA
     const int dk = a.dk, dv = a.dv, nq = a.nq, nkv = a.nkv, page_size = a.page_size, window = a.window;
     const int n_pieces = (dk + PF - 1) / PF;
     const int krow = n_pieces * PF + E;           // padded LDS row of keys and of queries
+    const int k_pieces = dk / E;                  // 16-byte pieces of a key
     T* q_s = reinterpret_cast<T*>(window_smem);
     T* k_s = q_s + ROWS * krow;
     T* v_s = k_s + KT * krow;
@@ -283,19 +288,35 @@ __global__ __launch_bounds__(64 * RT) void window_attention_tiled_kernel(WindowA
         lo_row[w] = (window > 0 && valid[w]) ? max(0, p_row[w] - window + 1) : 0;
     }
 
-    // queries into LDS, zeros beyond the key size and in rows that belong to no token
+    // queries into LDS, zeros beyond the key size and in rows that belong to no token; the pads of the key rows and the
+    // value rows beyond the value size are zeroed once, the chunks never write there
     {
         const int pieces = krow / E;
-        for (int idx = tid; idx < ROWS * pieces; idx += THREADS) {
-            const int row = idx / pieces, c = idx % pieces;
-            const int rr = blk_first + row;
-            w_u32x4 v = w_u32x4{0u, 0u, 0u, 0u};
-            if (rr < rows && c * E < dk) {
-                const int t2 = qs + rr / group_size, h2 = kh * group_size + rr % group_size;
-                v = *reinterpret_cast<const w_u32x4*>(q + (static_cast<size_t>(t2) * nq + h2) * dk + c * E);
+        for (int base = tid; base < ROWS * pieces; base += THREADS * U) {
+            w_u32x4 regs[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int idx = base + u * THREADS;
+                const int row = idx / pieces, c = idx % pieces;
+                const int rr = blk_first + row;
+                regs[u] = w_u32x4{0u, 0u, 0u, 0u};
+                if (idx < ROWS * pieces && rr < rows && c * E < dk) {
+                    const int t2 = qs + rr / group_size, h2 = kh * group_size + rr % group_size;
+                    regs[u] = *reinterpret_cast<const w_u32x4*>(q + (static_cast<size_t>(t2) * nq + h2) * dk + c * E);
+                }
             }
-            *reinterpret_cast<w_u32x4*>(q_s + row * krow + c * E) = v;
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int idx = base + u * THREADS;
+                if (idx < ROWS * pieces) *reinterpret_cast<w_u32x4*>(q_s + (idx / pieces) * krow + (idx % pieces) * E) = regs[u];
+            }
         }
+        for (int idx = tid; idx < KT * (pieces - k_pieces); idx += THREADS)
+            *reinterpret_cast<w_u32x4*>(k_s + (idx / (pieces - k_pieces)) * krow + (k_pieces + idx % (pieces - k_pieces)) * E) =
+                w_u32x4{0u, 0u, 0u, 0u};
+        constexpr int VPIECES = VROW / E;
+        for (int idx = tid; idx < DT * 16 * VPIECES; idx += THREADS)
+            if (idx / VPIECES >= dv) *reinterpret_cast<w_u32x4*>(v_s + (idx / VPIECES) * VROW + (idx % VPIECES) * E) = w_u32x4{0u, 0u, 0u, 0u};
     }
 
     w_f32x4 o[RW][DT];
@@ -309,90 +330,94 @@ __global__ __launch_bounds__(64 * RT) void window_attention_tiled_kernel(WindowA
     }
     const float scale = a.scale;
     constexpr float kLog2e = 1.4426950408889634f;
+    const bool wave_active = blk_first + wave * RW * 16 < rows;      // a wavefront without rows only helps to stage
 
+    // A chunk's keys [KT][dk] and values, transposed [dv][KT], travel through registers: the loads of the chunk after
+    // this one are issued before this one's products and stored to LDS behind them.  What no row of the workgroup sees
+    // is zeros.  A thread holds at most KU pieces of 16 bytes of keys (dk <= 256) and VU of values.
+    constexpr int VKP = KT / E;   // 16-byte pieces of a value row
+    w_u32x4 k_regs[KU], v_regs[VU];
+    const int k_total = KT * k_pieces, v_total = dv * VKP;
+    auto fetch = [&](int c) {
+        const bool any = c < c_end;
+        const int tile = c < kept_chunks ? c : t_begin + (c - kept_chunks);
+        const int key0 = tile * KT;
+        long k_page[KU], v_page[VU];
+#pragma unroll
+        for (int u = 0; u < KU; ++u) {
+            const int idx = tid + u * THREADS;
+            const int j = key0 + idx / k_pieces;
+            k_page[u] = -1;
+            if (any && idx < k_total && j <= p_max && (j >= lo_blk || j < keep)) k_page[u] = table[j / page_size];
+        }
+#pragma unroll
+        for (int u = 0; u < VU; ++u) {
+            const int idx = tid + u * THREADS;
+            const int j = key0 + (idx % VKP) * E;
+            v_page[u] = -1;
+            if (any && idx < v_total && j <= p_max && (j + E - 1 >= lo_blk || j < keep)) v_page[u] = table[j / page_size];
+        }
+#pragma unroll
+        for (int u = 0; u < KU; ++u) {
+            const int idx = tid + u * THREADS;
+            const int j = key0 + idx / k_pieces, cc = idx % k_pieces;
+            k_regs[u] = w_u32x4{0u, 0u, 0u, 0u};
+            if (k_page[u] >= 0)
+                k_regs[u] = *reinterpret_cast<const w_u32x4*>(k_cache + ((k_page[u] * nkv + kh) * page_size + j % page_size) * dk + cc * E);
+        }
+#pragma unroll
+        for (int u = 0; u < VU; ++u) {
+            const int idx = tid + u * THREADS;
+            const int f = idx / VKP, j = key0 + (idx % VKP) * E;
+            w_u32x4 v = w_u32x4{0u, 0u, 0u, 0u};
+            if (v_page[u] >= 0) {
+                v = *reinterpret_cast<const w_u32x4*>(v_cache + ((v_page[u] * nkv + kh) * dv + f) * page_size + j % page_size);
+                if (j + E > kv) {         // places of the page that no token has written yet may hold anything
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        if constexpr (sizeof(T) == 4) {
+                            if (j + e >= kv) v[e] = 0u;
+                        } else {
+                            if (j + 2 * e >= kv) v[e] = 0u;
+                            else if (j + 2 * e + 1 >= kv) v[e] &= 0x0000ffffu;
+                        }
+                    }
+                }
+            }
+            v_regs[u] = v;
+        }
+    };
+    auto stash = [&]() {
+#pragma unroll
+        for (int u = 0; u < KU; ++u) {
+            const int idx = tid + u * THREADS;
+            if (idx < k_total) *reinterpret_cast<w_u32x4*>(k_s + (idx / k_pieces) * krow + (idx % k_pieces) * E) = k_regs[u];
+        }
+#pragma unroll
+        for (int u = 0; u < VU; ++u) {
+            const int idx = tid + u * THREADS;
+            if (idx >= v_total) continue;
+            const int f = idx / VKP, v_key = (idx % VKP) * E;
+            if constexpr (sizeof(T) == 4) {
+                *reinterpret_cast<w_u32x4*>(v_s + f * VROW + v_key) = v_regs[u];
+            } else {
+                // in the order in which a lane takes them: within 32 keys (quarter of the wavefront, tile, key)
+                const int v_pos = (v_key / 32) * 32 + ((v_key % 16) / 4) * 8 + ((v_key % 32) / 16) * 4;
+                *reinterpret_cast<w_u32x2*>(v_s + f * VROW + v_pos) = w_u32x2{v_regs[u].x, v_regs[u].y};
+                *reinterpret_cast<w_u32x2*>(v_s + f * VROW + v_pos + 8) = w_u32x2{v_regs[u].z, v_regs[u].w};
+            }
+        }
+    };
+
+    fetch(c_begin);
     for (int c = c_begin; c < c_end; ++c) {
         const int tile = c < kept_chunks ? c : t_begin + (c - kept_chunks);
         const int key0 = tile * KT;
         __syncthreads();                  // the chunk before is read (and, the first time, the queries are written)
-        // ---- stage the chunk: keys [KT][dk], values transposed [dv][KT]; what no row of the workgroup sees is zeros.
-        // U loads of a thread are issued before the first is stored.
-        {
-            const int pieces = krow / E;
-            const int total = KT * pieces;
-            for (int base = tid; base < total; base += THREADS * U) {
-                w_u32x4 regs[U];
-                long pages[U];
-#pragma unroll
-                for (int u = 0; u < U; ++u) {
-                    const int idx = base + u * THREADS;
-                    const int j = key0 + idx / pieces, cc = idx % pieces;
-                    pages[u] = -1;
-                    if (idx < total && j <= p_max && (j >= lo_blk || j < keep) && cc * E < dk) pages[u] = table[j / page_size];
-                }
-#pragma unroll
-                for (int u = 0; u < U; ++u) {
-                    const int idx = base + u * THREADS;
-                    const int j = key0 + idx / pieces, cc = idx % pieces;
-                    regs[u] = w_u32x4{0u, 0u, 0u, 0u};
-                    if (pages[u] >= 0)
-                        regs[u] = *reinterpret_cast<const w_u32x4*>(k_cache + ((pages[u] * nkv + kh) * page_size + j % page_size) * dk + cc * E);
-                }
-#pragma unroll
-                for (int u = 0; u < U; ++u) {
-                    const int idx = base + u * THREADS;
-                    if (idx < total) *reinterpret_cast<w_u32x4*>(k_s + (idx / pieces) * krow + (idx % pieces) * E) = regs[u];
-                }
-            }
-            constexpr int VKP = KT / E;   // 16-byte pieces of a value row
-            constexpr int VTOTAL = DT * 16 * VKP;
-            for (int base = tid; base < VTOTAL; base += THREADS * U) {
-                w_u32x4 regs[U];
-                long pages[U];
-#pragma unroll
-                for (int u = 0; u < U; ++u) {
-                    const int idx = base + u * THREADS;
-                    const int f = idx / VKP, j = key0 + (idx % VKP) * E;
-                    pages[u] = -1;
-                    if (idx < VTOTAL && f < dv && j <= p_max && (j + E - 1 >= lo_blk || j < keep)) pages[u] = table[j / page_size];
-                }
-#pragma unroll
-                for (int u = 0; u < U; ++u) {
-                    const int idx = base + u * THREADS;
-                    const int f = idx / VKP, j = key0 + (idx % VKP) * E;
-                    w_u32x4 v = w_u32x4{0u, 0u, 0u, 0u};
-                    if (pages[u] >= 0) {
-                        v = *reinterpret_cast<const w_u32x4*>(v_cache + ((pages[u] * nkv + kh) * dv + f) * page_size + j % page_size);
-                        if (j + E > kv) {         // places of the page that no token has written yet may hold anything
-#pragma unroll
-                            for (int e = 0; e < 4; ++e) {
-                                if constexpr (sizeof(T) == 4) {
-                                    if (j + e >= kv) v[e] = 0u;
-                                } else {
-                                    if (j + 2 * e >= kv) v[e] = 0u;
-                                    else if (j + 2 * e + 1 >= kv) v[e] &= 0x0000ffffu;
-                                }
-                            }
-                        }
-                    }
-                    regs[u] = v;
-                }
-#pragma unroll
-                for (int u = 0; u < U; ++u) {
-                    const int idx = base + u * THREADS;
-                    if (idx >= VTOTAL) continue;
-                    const int f = idx / VKP, v_key = (idx % VKP) * E;
-                    if constexpr (sizeof(T) == 4) {
-                        *reinterpret_cast<w_u32x4*>(v_s + f * VROW + v_key) = regs[u];
-                    } else {
-                        // in the order in which a lane takes them: within 32 keys (quarter of the wavefront, tile, key)
-                        const int v_pos = (v_key / 32) * 32 + ((v_key % 16) / 4) * 8 + ((v_key % 32) / 16) * 4;
-                        *reinterpret_cast<w_u32x2*>(v_s + f * VROW + v_pos) = w_u32x2{regs[u].x, regs[u].y};
-                        *reinterpret_cast<w_u32x2*>(v_s + f * VROW + v_pos + 8) = w_u32x2{regs[u].z, regs[u].w};
-                    }
-                }
-            }
-        }
+        stash();
         __syncthreads();
+        fetch(c + 1);                     // in flight while this chunk is computed; behind the last chunk nothing is read
+        if (!wave_active) continue;
         // ---- scores of this wavefront's rows against the chunk's keys: a key operand serves all of its row tiles
         w_f32x4 acc[RW][NKT];
         const T* ks = k_s + lj * krow + lg * E;
@@ -565,12 +590,11 @@ static int launch_tiled(const WindowArgs& a, int max_rows, hipStream_t s) {
     return EGPT_OK;
 }
 
-// row_tiles: 1 (a wavefront with 16 rows), 4 (four wavefronts with 16 rows each) or 8 (four with 32 rows each)
+// row_tiles: 4 (four wavefronts with 16 rows each) or 8 (with 32 rows each)
 template <typename T, int DT>
 static int launch_tiled_for_rows(const WindowArgs& a, int max_rows, int row_tiles, hipStream_t s) {
     if (row_tiles == 8) return launch_tiled<T, DT, 4, 2>(a, max_rows, s);
-    if (row_tiles == 4) return launch_tiled<T, DT, 4, 1>(a, max_rows, s);
-    return launch_tiled<T, DT, 1, 1>(a, max_rows, s);
+    return launch_tiled<T, DT, 4, 1>(a, max_rows, s);
 }
 
 template <typename T>
@@ -625,11 +649,11 @@ extern "C" int egpt_window_attention_tiled(const void* q, void* out, float* part
     if (!q || !out || !k_cache || !v_cache || !block_table || !q_start || !q_len || !kv_len) return EGPT_BAD_ARGUMENT;
     if (n_seqs <= 0 || n_tokens < 0 || nq <= 0 || nkv <= 0 || nq % nkv != 0 || dk <= 0 || dv <= 0 || page_size <= 0 ||
         table_width <= 0 || window < 0 || keep_first < 0 || n_splits < 1 || (dtype != 0 && dtype != 1) ||
-        (row_tiles != 1 && row_tiles != 4 && row_tiles != 8))
+        (row_tiles != 4 && row_tiles != 8))
         return EGPT_BAD_ARGUMENT;
     if (n_splits > 1 && (!part_o || !part_ml)) return EGPT_BAD_ARGUMENT;
     const int e = dtype == 0 ? 4 : 8;
-    if (dk % e || dv % 16 || dv > 256 || page_size % 16 || nkv > 65535 || n_splits > 64) return EGPT_UNSUPPORTED_SIZE;
+    if (dk % e || dk > 256 || dv % 16 || dv > 256 || page_size % 16 || nkv > 65535 || n_splits > 64) return EGPT_UNSUPPORTED_SIZE;
     if (n_tokens == 0) return EGPT_OK;
     hipStream_t s = static_cast<hipStream_t>(stream);
     WindowArgs a;

@@ -965,21 +965,24 @@ class HipKernels(KernelBackend):
                   block_table.data_ptr(), width, q_start.data_ptr(), q_len.data_ptr(), kv_len.data_ptr(), b, t, nq, nkv,
                   dk, dv, page_size, float(scale), int(window), int(keep_first), self._ptr(sink), dt, self._stream())
 
-    wide_rows_from = 16384          # rows of a step from which the window attention gives a wavefront 32 of them
+    wide_rows_from = 16384          # rows of a step from which the window attention gives a wavefront 32 of them,
+    wide_rows_key_size = 192        # if its keys are wider than this
 
     @staticmethod
     def _window_attention_shape(t, b, nq, nkv, dk, dv, page_size, window, keep_first, max_q_len, max_kv_len, elem):
         """(row tiles per workgroup, splits of the keys) of the matrix-core window attention, or None where its sizes
-        are not covered.  Prompt portions: workgroups of 64 rows that walk their keys alone.  Steps whose requests
-        bring so few rows that one tile of 16 holds them (single tokens): one wavefront per workgroup, and the chunks
-        of keys that a row sees dealt over enough workgroups to fill the GPU, a chunk or more each."""
+        are not covered.  Steps of many rows: 32 rows to a wavefront.  Steps of so few rows that their workgroups do
+        not fill the GPU (single tokens, short portions): the chunks of keys that a workgroup's rows see are dealt
+        over several workgroups, a chunk or more each, and a second kernel folds their results."""
         e = 16 // elem
-        if dk % e or dv % 16 or dv > 256 or page_size % 16:
+        if dk % e or dk > 256 or dv % 16 or dv > 256 or page_size % 16:
             return None
         chunk = 64 if elem == 2 else 32
         group = nq // nkv
-        # many rows: 32 to a wavefront, which halves the reads of a chunk's keys and values from LDS per row
-        row_tiles = 1 if max_q_len * group <= 16 else 4 if t * group * nkv < HipKernels.wide_rows_from else 8
+        # (measured, us for a 2,048-token prompt behind nothing, 16 / 32 rows to a wavefront: 14 heads on 2 of 64 + 64, window
+        # 1,024: 70 / 73; 14 on 1 of 160 + 128: 96 / 137; 16 on 4 of 128 + 128, window 2,048: 162 / 191; 16 on 1 of 256 + 192:
+        # 310 / 274)
+        row_tiles = 8 if dk > HipKernels.wide_rows_key_size and t * group * nkv >= HipKernels.wide_rows_from else 4
         krow = -(-dk // (4 * e)) * 4 * e + e
         dv_tiles = next(n for n in (2, 4, 6, 8, 12, 16) if n * 16 >= dv)
         lds = lambda tiles: ((16 * tiles + chunk) * krow + dv_tiles * 16 * (chunk + e)) * elem
@@ -988,10 +991,10 @@ class HipKernels(KernelBackend):
         if lds(row_tiles) > 160 * 1024:
             return None
         workgroups = (-(-t * group // (16 * row_tiles)) + b) * nkv
-        span = min(max_kv_len, window + chunk) if window else max_kv_len
+        span = min(max_kv_len, window + min(max_q_len, 64) + chunk) if window else max_kv_len
         chunks = -(-span // chunk) + (-(-min(keep_first, max_kv_len) // chunk) if window else 0)
         n_splits = 1
-        if row_tiles == 1 and workgroups < 512:
+        if workgroups < 256 and chunks > 1:
             n_splits = max(1, min(chunks, -(-512 // workgroups), 64))
         return row_tiles, n_splits
 

@@ -219,8 +219,8 @@ def test_attention_with_32_rows_to_a_wavefront(k, dtype, nq, nkv, dk, dv, window
     scale = 1.7 / math.sqrt(dk)
     k_cache, v_cache, table = paged(keys, values, ps, dtype, seed=85)
     want = plain_attention(q, keys, values, 0, scale, window, keep_first, sink)
-    before = HipKernels.wide_rows_from
-    HipKernels.wide_rows_from = 0
+    before = HipKernels.wide_rows_from, HipKernels.wide_rows_key_size
+    HipKernels.wide_rows_from = HipKernels.wide_rows_key_size = 0
     try:
         assert HipKernels._window_attention_shape(n, 1, nq, nkv, dk, dv, ps, window, keep_first, n, n, q.element_size())[0] == 8
         got = run_attention(k, q, k_cache, v_cache, table, n, ps, scale, window, keep_first, sink, dv)
@@ -228,7 +228,7 @@ def test_attention_with_32_rows_to_a_wavefront(k, dtype, nq, nkv, dk, dv, window
         got = run_attention(k, q[200:301], k_cache, v_cache, table, 301, ps, scale, window, keep_first, sink, dv)
         close(got, want[200:301], dtype, "a portion")
     finally:
-        HipKernels.wide_rows_from = before
+        HipKernels.wide_rows_from, HipKernels.wide_rows_key_size = before
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
