@@ -122,15 +122,18 @@ int egpt_gemm_skinny_attn(const float* part_o, const float* part_ml, int a_split
 // and w bfloat16 [2 * inter][k] (gate rows, then up rows); k % 8 == 0.
 int egpt_gemm_gate_up_swiglu(const void* x, const void* w, void* out, int m, int inter, int k, int groups, void* stream);
 // ---- mixers that norm or rotate single heads (head_prep.hip), and their attention (attention_window.hip)
-// out float32 [n_tokens][hidden] = table[id] / sqrt(mean(table[id]^2) + eps) * weight: an embedding with its norm, as
-// the residual stream.
-int egpt_embed_rmsnorm(const int32_t* ids, const void* table, const void* weight, float eps, float* out, int n_tokens,
-                       int hidden, int vocab, int dtype, void* stream);
+// out [n_tokens][hidden] = table[id] / sqrt(mean(table[id]^2) + eps) * weight: an embedding with its norm, as the
+// residual stream (float32, or fixed point with fixed != 0).  In the three functions below row_ss (may be null)
+// float32 [ss_splits][n_tokens] says that the product (float32 partial sums) still lacks each row's factor
+// 1 / sqrt(sum_s row_ss[s][t] / hidden + norm_eps), as a product with the norm folded in leaves it.
+int egpt_embed_rmsnorm(const int32_t* ids, const void* table, const void* weight, float eps, void* out, int fixed,
+                       int n_tokens, int hidden, int vocab, int dtype, void* stream);
 // proj rows [nq heads of dk | nkv heads of dk | nkv heads of dv] (n_splits > 0: float32 partial sums).  Query and key
 // heads are divided by their root mean square and multiplied by q_weight / k_weight [dk] (null: the heads pass as they
 // are), value heads are divided by theirs if norm_values != 0.  Queries to q_out [n_tokens][nq * dk]; keys
 // [pages][nkv][page_size][dk] and values [pages][nkv][dv][page_size] to slots[t] (null: not stored).
-int egpt_head_norm_store(const void* proj, int n_splits, void* q_out, const void* q_weight, const void* k_weight, float eps,
+int egpt_head_norm_store(const void* proj, int n_splits, const float* row_ss, int ss_splits, int hidden, float norm_eps,
+                         void* q_out, const void* q_weight, const void* k_weight, float eps,
                          int norm_values, const int32_t* slots, void* k_cache, void* v_cache, int n_tokens, int nq,
                          int nkv, int dk, int dv, int page_size, int dtype, void* stream);
 // proj rows of row_width values: [nq heads of (dim | rot) | rank | rot | ...].  q_plain [n_tokens][nq][dim] takes the
@@ -138,13 +141,15 @@ int egpt_head_norm_store(const void* proj, int n_splits, void* q_out, const void
 // latent (normed with c_weight [rank]) and the rotated shared key are stored as key [pages][1][page_size][rank + rot],
 // the latent also as value [pages][1][rank][page_size].  cos_sin float32 [n_tokens][rot_dims / 2][2], multiplied by
 // mag; pairs (2i, 2i + 1) of the first rot_dims places of a rotated part are rotated.
-int egpt_latent_prep(const void* proj, int n_splits, int row_width, void* q_plain, void* q_full, const void* c_weight,
+int egpt_latent_prep(const void* proj, int n_splits, const float* row_ss, int ss_splits, int hidden, float norm_eps,
+                     int row_width, void* q_plain, void* q_full, const void* c_weight,
                      float eps, const float* cos_sin, float mag, int rot_dims, const int32_t* slots, void* k_cache,
                      void* v_cache, int n_tokens, int nq, int dim, int rot, int rank, int page_size, int dtype,
                      void* stream);
 // out [n_tokens][n] = x * sigmoid(gate[:, gate_off : gate_off + n]); x [n_tokens][n], or with heads > 0
 // [heads][n_tokens][n / heads]; gate: rows of gate_width values (gate_splits > 0: float32 partial sums).
-int egpt_sigmoid_gate(const void* x, int heads, const void* gate, int gate_splits, int gate_width, int gate_off, void* out,
+int egpt_sigmoid_gate(const void* x, int heads, const void* gate, int gate_splits, const float* row_ss, int ss_splits,
+                      int hidden, float norm_eps, int gate_width, int gate_off, void* out,
                       int n_tokens, int n, int dtype, void* stream);
 // Attention with key size dk and value size dv, a window that keeps the first keep_first tokens visible, and an
 // optional sink per query head (float32 [nq], null: none) in the softmax's denominator.  q [n_tokens][nq][dk],

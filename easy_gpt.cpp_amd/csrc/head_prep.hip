@@ -11,14 +11,28 @@
 
 namespace egpt {
 
+// A product whose x operand was (h * norm weight) still lacks each row's factor 1 / sqrt(sum_s ss[s][row] / hidden + eps):
+// the sums of squares arrive beside it (null: the product is complete).
+struct RowFactor {
+    const float* ss;
+    int splits, n_rows, hidden;
+    float eps;
+    __device__ __forceinline__ float of(int row) const {
+        if (ss == nullptr) return 1.0f;
+        float total = 0.f;
+        for (int s = 0; s < splits; ++s) total += ss[static_cast<size_t>(s) * n_rows + row];
+        return inv_rms(total, 1.0f / static_cast<float>(hidden), eps);
+    }
+};
+
 constexpr int kMaxHeadWidth = 1024;                   // the widest head (or latent) these kernels take
 constexpr int kOwn = kMaxHeadWidth / kWave;           // values of it that a lane keeps
 
-// x[t, :] = E[id_t, :] / sqrt(mean(E[id_t, :]^2) + eps) * w, written as the float32 residual stream.
-template <typename T>
+// x[t, :] = E[id_t, :] / sqrt(mean(E[id_t, :]^2) + eps) * w, written as the residual stream (float32 or fixed point).
+template <typename T, typename R>
 __global__ __launch_bounds__(256) void embed_rmsnorm_kernel(const int32_t* __restrict__ ids, const T* __restrict__ table,
                                                             const T* __restrict__ weight, float eps,
-                                                            float* __restrict__ out, int hidden, int vocab) {
+                                                            R* __restrict__ out, int hidden, int vocab) {
     __shared__ float scratch[16];
     const int t = blockIdx.x;
     int id = ids[t];
@@ -31,8 +45,8 @@ __global__ __launch_bounds__(256) void embed_rmsnorm_kernel(const int32_t* __res
     }
     ss = block_sum(ss, scratch);
     const float inv = inv_rms(ss, 1.0f / static_cast<float>(hidden), eps);
-    float* o = out + static_cast<size_t>(t) * hidden;
-    for (int j = threadIdx.x; j < hidden; j += blockDim.x) o[j] = to_float(row[j]) * inv * to_float(weight[j]);
+    R* o = out + static_cast<size_t>(t) * hidden;
+    for (int j = threadIdx.x; j < hidden; j += blockDim.x) residual_store(o + j, to_float(row[j]) * inv * to_float(weight[j]));
 }
 
 // One wavefront per (token, head) of a product row [nq heads of dk | nkv heads of dk | nkv heads of dv]: a query or
@@ -41,8 +55,8 @@ __global__ __launch_bounds__(256) void embed_rmsnorm_kernel(const int32_t* __res
 // to q_out [T][nq * dk]; keys and values to the pages at slots[t] (slots null: nothing is stored).
 template <typename T>
 __global__ __launch_bounds__(kWave) void head_norm_store_kernel(
-    ProductView<T> proj, T* __restrict__ q_out, const T* __restrict__ q_weight, const T* __restrict__ k_weight, float eps,
-    int norm_values, const int32_t* __restrict__ slots, T* __restrict__ k_cache, T* __restrict__ v_cache, int nq, int nkv,
+    ProductView<T> proj, RowFactor factor, T* __restrict__ q_out, const T* __restrict__ q_weight,
+    const T* __restrict__ k_weight, float eps, int norm_values, const int32_t* __restrict__ slots, T* __restrict__ k_cache, T* __restrict__ v_cache, int nq, int nkv,
     int dk, int dv, int page_size) {
     const int t = blockIdx.x, hh = blockIdx.y, lane = threadIdx.x;
     const int row_width = (nq + nkv) * dk + nkv * dv;
@@ -54,12 +68,13 @@ __global__ __launch_bounds__(kWave) void head_norm_store_kernel(
     const T* weight = kind == 0 ? q_weight : (kind == 1 ? k_weight : nullptr);
     const bool normed = kind == 2 ? norm_values != 0 : weight != nullptr;
     const size_t base = static_cast<size_t>(t) * row_width + in_off;
+    const float rf = factor.of(t);
     float v[kOwn];
     float ss = 0.f;
 #pragma unroll
     for (int r = 0; r < kOwn; ++r) {
         const int d = lane + r * kWave;
-        v[r] = d < width ? proj.at(base + d) : 0.f;
+        v[r] = d < width ? proj.at(base + d) * rf : 0.f;
         ss = fmaf(v[r], v[r], ss);
     }
     float inv = 1.0f;
@@ -95,26 +110,27 @@ __global__ __launch_bounds__(kWave) void head_norm_store_kernel(
 // cos_sin [T][rot_dims / 2][2]; both are multiplied by mag; places from rot_dims on pass unchanged.
 template <typename T>
 __global__ __launch_bounds__(kWave) void latent_prep_kernel(
-    ProductView<T> proj, int row_width, T* __restrict__ q_plain, T* __restrict__ q_full, const T* __restrict__ c_weight,
-    float eps, const float* __restrict__ cos_sin, float mag, int rot_dims, const int32_t* __restrict__ slots,
+    ProductView<T> proj, RowFactor factor, int row_width, T* __restrict__ q_plain, T* __restrict__ q_full,
+    const T* __restrict__ c_weight, float eps, const float* __restrict__ cos_sin, float mag, int rot_dims, const int32_t* __restrict__ slots,
     T* __restrict__ k_cache, T* __restrict__ v_cache, int nq, int dim, int rot, int rank, int page_size) {
     const int t = blockIdx.x, hh = blockIdx.y, lane = threadIdx.x;
     const size_t row = static_cast<size_t>(t) * row_width;
     const float* cs = cos_sin + static_cast<size_t>(t) * rot_dims;      // (rot_dims / 2) pairs of (cos, sin)
     const int dk = rank + rot;
+    const float rf = factor.of(t);
     if (hh < nq) {
         const size_t base = row + static_cast<size_t>(hh) * (dim + rot);
         for (int d = lane; d < dim; d += kWave)
-            q_plain[(static_cast<size_t>(t) * nq + hh) * dim + d] = from_float<T>(proj.at(base + d));
+            q_plain[(static_cast<size_t>(t) * nq + hh) * dim + d] = from_float<T>(proj.at(base + d) * rf);
         T* dst = q_full + (static_cast<size_t>(t) * nq + hh) * dk + rank;
         for (int i = lane; i < rot / 2; i += kWave) {
-            const float u = proj.at(base + dim + 2 * i), w = proj.at(base + dim + 2 * i + 1);
+            const float u = proj.at(base + dim + 2 * i) * rf, w = proj.at(base + dim + 2 * i + 1) * rf;
             float ru = u, rw = w;
             if (2 * i + 1 < rot_dims) rotate_pair(u, w, cs[2 * i] * mag, cs[2 * i + 1] * mag, ru, rw);
             dst[2 * i] = from_float<T>(ru);
             dst[2 * i + 1] = from_float<T>(rw);
         }
-        if ((rot & 1) && lane == 0) dst[rot - 1] = from_float<T>(proj.at(base + dim + rot - 1));
+        if ((rot & 1) && lane == 0) dst[rot - 1] = from_float<T>(proj.at(base + dim + rot - 1) * rf);
         return;
     }
     if (slots == nullptr) return;
@@ -124,7 +140,7 @@ __global__ __launch_bounds__(kWave) void latent_prep_kernel(
 #pragma unroll
     for (int r = 0; r < kOwn; ++r) {
         const int d = lane + r * kWave;
-        v[r] = d < rank ? proj.at(base + d) : 0.f;
+        v[r] = d < rank ? proj.at(base + d) * rf : 0.f;
         ss = fmaf(v[r], v[r], ss);
     }
     const float inv = inv_rms(wave_sum(ss), 1.0f / static_cast<float>(rank), eps);
@@ -141,20 +157,20 @@ __global__ __launch_bounds__(kWave) void latent_prep_kernel(
         vdst[static_cast<long>(d) * page_size] = y;
     }
     for (int i = lane; i < rot / 2; i += kWave) {
-        const float u = proj.at(base + rank + 2 * i), w = proj.at(base + rank + 2 * i + 1);
+        const float u = proj.at(base + rank + 2 * i) * rf, w = proj.at(base + rank + 2 * i + 1) * rf;
         float ru = u, rw = w;
         if (2 * i + 1 < rot_dims) rotate_pair(u, w, cs[2 * i] * mag, cs[2 * i + 1] * mag, ru, rw);
         kdst[rank + 2 * i] = from_float<T>(ru);
         kdst[rank + 2 * i + 1] = from_float<T>(rw);
     }
-    if ((rot & 1) && lane == 0) kdst[rank + rot - 1] = from_float<T>(proj.at(base + rank + rot - 1));
+    if ((rot & 1) && lane == 0) kdst[rank + rot - 1] = from_float<T>(proj.at(base + rank + rot - 1) * rf);
 }
 
 // out[t][n] = x[t][n] * sigmoid(g[t][gate_off + n]); x lies [T][N], or with heads > 0 head by head [heads][T][N / heads]
 // (what a product batched over heads leaves).  g: columns of a product row of width gate_width.
 template <typename T>
 __global__ __launch_bounds__(256) void sigmoid_gate_kernel(const T* __restrict__ x, int heads, ProductView<T> g,
-                                                           int gate_width, int gate_off, T* __restrict__ out,
+                                                           RowFactor factor, int gate_width, int gate_off, T* __restrict__ out,
                                                            int n_tokens, int n) {
     const size_t idx = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     if (idx >= static_cast<size_t>(n_tokens) * n) return;
@@ -164,7 +180,7 @@ __global__ __launch_bounds__(256) void sigmoid_gate_kernel(const T* __restrict__
         const int per = n / heads;
         src = (static_cast<size_t>(c / per) * n_tokens + t) * per + c % per;
     }
-    const float gate = g.at(static_cast<size_t>(t) * gate_width + gate_off + c);
+    const float gate = g.at(static_cast<size_t>(t) * gate_width + gate_off + c) * factor.of(t);
     out[idx] = from_float<T>(to_float(x[src]) * (1.0f / (1.0f + expf(-gate))));
 }
 
@@ -182,23 +198,30 @@ static ProductView<T> view_of(const void* p, int n_splits, size_t split_stride) 
 
 using namespace egpt;
 
-extern "C" int egpt_embed_rmsnorm(const int32_t* ids, const void* table, const void* weight, float eps, float* out,
-                                  int n_tokens, int hidden, int vocab, int dtype, void* stream) {
+extern "C" int egpt_embed_rmsnorm(const int32_t* ids, const void* table, const void* weight, float eps, void* out,
+                                  int fixed, int n_tokens, int hidden, int vocab, int dtype, void* stream) {
     if (!ids || !table || !weight || !out || n_tokens < 0 || hidden <= 0 || vocab <= 0 || (dtype != 0 && dtype != 1))
         return EGPT_BAD_ARGUMENT;
     if (n_tokens == 0) return EGPT_OK;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if (dtype == 0)
-        embed_rmsnorm_kernel<<<n_tokens, 256, 0, s>>>(ids, static_cast<const float*>(table),
-                                                      static_cast<const float*>(weight), eps, out, hidden, vocab);
+    if (dtype == 0 && !fixed)
+        embed_rmsnorm_kernel<<<n_tokens, 256, 0, s>>>(ids, static_cast<const float*>(table), static_cast<const float*>(weight),
+                                                      eps, static_cast<float*>(out), hidden, vocab);
+    else if (dtype == 0)
+        embed_rmsnorm_kernel<<<n_tokens, 256, 0, s>>>(ids, static_cast<const float*>(table), static_cast<const float*>(weight),
+                                                      eps, static_cast<fixed_t*>(out), hidden, vocab);
+    else if (!fixed)
+        embed_rmsnorm_kernel<<<n_tokens, 256, 0, s>>>(ids, static_cast<const bf16_t*>(table), static_cast<const bf16_t*>(weight),
+                                                      eps, static_cast<float*>(out), hidden, vocab);
     else
-        embed_rmsnorm_kernel<<<n_tokens, 256, 0, s>>>(ids, static_cast<const bf16_t*>(table),
-                                                      static_cast<const bf16_t*>(weight), eps, out, hidden, vocab);
+        embed_rmsnorm_kernel<<<n_tokens, 256, 0, s>>>(ids, static_cast<const bf16_t*>(table), static_cast<const bf16_t*>(weight),
+                                                      eps, static_cast<fixed_t*>(out), hidden, vocab);
     EGPT_CHECK_LAUNCH();
     return EGPT_OK;
 }
 
-extern "C" int egpt_head_norm_store(const void* proj, int n_splits, void* q_out, const void* q_weight,
+extern "C" int egpt_head_norm_store(const void* proj, int n_splits, const float* row_ss, int ss_splits, int hidden,
+                                    float norm_eps, void* q_out, const void* q_weight,
                                     const void* k_weight, float eps, int norm_values, const int32_t* slots,
                                     void* k_cache, void* v_cache, int n_tokens, int nq, int nkv, int dk, int dv,
                                     int page_size, int dtype, void* stream) {
@@ -209,23 +232,26 @@ extern "C" int egpt_head_norm_store(const void* proj, int n_splits, void* q_out,
     if (dk > kMaxHeadWidth || dv > kMaxHeadWidth || nq + 2 * nkv > 65535) return EGPT_UNSUPPORTED_SIZE;
     if (n_tokens == 0) return EGPT_OK;
     hipStream_t s = static_cast<hipStream_t>(stream);
+    if (row_ss && (n_splits < 1 || ss_splits < 1 || hidden <= 0)) return EGPT_BAD_ARGUMENT;
+    const RowFactor factor{row_ss, ss_splits, n_tokens, hidden, norm_eps};
     const size_t stride = static_cast<size_t>(n_tokens) * ((nq + nkv) * dk + nkv * dv);
     dim3 grid(n_tokens, nq + 2 * nkv);
     if (dtype == 0)
         head_norm_store_kernel<float><<<grid, kWave, 0, s>>>(
-            view_of<float>(proj, n_splits, stride), static_cast<float*>(q_out), static_cast<const float*>(q_weight),
+            view_of<float>(proj, n_splits, stride), factor, static_cast<float*>(q_out), static_cast<const float*>(q_weight),
             static_cast<const float*>(k_weight), eps, norm_values, slots, static_cast<float*>(k_cache),
             static_cast<float*>(v_cache), nq, nkv, dk, dv, page_size);
     else
         head_norm_store_kernel<bf16_t><<<grid, kWave, 0, s>>>(
-            view_of<bf16_t>(proj, n_splits, stride), static_cast<bf16_t*>(q_out), static_cast<const bf16_t*>(q_weight),
+            view_of<bf16_t>(proj, n_splits, stride), factor, static_cast<bf16_t*>(q_out), static_cast<const bf16_t*>(q_weight),
             static_cast<const bf16_t*>(k_weight), eps, norm_values, slots, static_cast<bf16_t*>(k_cache),
             static_cast<bf16_t*>(v_cache), nq, nkv, dk, dv, page_size);
     EGPT_CHECK_LAUNCH();
     return EGPT_OK;
 }
 
-extern "C" int egpt_latent_prep(const void* proj, int n_splits, int row_width, void* q_plain, void* q_full,
+extern "C" int egpt_latent_prep(const void* proj, int n_splits, const float* row_ss, int ss_splits, int hidden,
+                                float norm_eps, int row_width, void* q_plain, void* q_full,
                                 const void* c_weight, float eps, const float* cos_sin, float mag, int rot_dims,
                                 const int32_t* slots, void* k_cache, void* v_cache, int n_tokens, int nq, int dim,
                                 int rot, int rank, int page_size, int dtype, void* stream) {
@@ -238,39 +264,44 @@ extern "C" int egpt_latent_prep(const void* proj, int n_splits, int row_width, v
     if (rank > kMaxHeadWidth || nq + 1 > 65535) return EGPT_UNSUPPORTED_SIZE;
     if (n_tokens == 0) return EGPT_OK;
     hipStream_t s = static_cast<hipStream_t>(stream);
+    if (row_ss && (n_splits < 1 || ss_splits < 1 || hidden <= 0)) return EGPT_BAD_ARGUMENT;
+    const RowFactor factor{row_ss, ss_splits, n_tokens, hidden, norm_eps};
     const size_t stride = static_cast<size_t>(n_tokens) * row_width;
     dim3 grid(n_tokens, nq + 1);
     if (dtype == 0)
         latent_prep_kernel<float><<<grid, kWave, 0, s>>>(
-            view_of<float>(proj, n_splits, stride), row_width, static_cast<float*>(q_plain), static_cast<float*>(q_full),
+            view_of<float>(proj, n_splits, stride), factor, row_width, static_cast<float*>(q_plain), static_cast<float*>(q_full),
             static_cast<const float*>(c_weight), eps, cos_sin, mag, rot_dims, slots, static_cast<float*>(k_cache),
             static_cast<float*>(v_cache), nq, dim, rot, rank, page_size);
     else
         latent_prep_kernel<bf16_t><<<grid, kWave, 0, s>>>(
-            view_of<bf16_t>(proj, n_splits, stride), row_width, static_cast<bf16_t*>(q_plain),
+            view_of<bf16_t>(proj, n_splits, stride), factor, row_width, static_cast<bf16_t*>(q_plain),
             static_cast<bf16_t*>(q_full), static_cast<const bf16_t*>(c_weight), eps, cos_sin, mag, rot_dims, slots,
             static_cast<bf16_t*>(k_cache), static_cast<bf16_t*>(v_cache), nq, dim, rot, rank, page_size);
     EGPT_CHECK_LAUNCH();
     return EGPT_OK;
 }
 
-extern "C" int egpt_sigmoid_gate(const void* x, int heads, const void* gate, int gate_splits, int gate_width,
+extern "C" int egpt_sigmoid_gate(const void* x, int heads, const void* gate, int gate_splits, const float* row_ss,
+                                 int ss_splits, int hidden, float norm_eps, int gate_width,
                                  int gate_off, void* out, int n_tokens, int n, int dtype, void* stream) {
     if (!x || !gate || !out || n_tokens < 0 || n <= 0 || heads < 0 || (heads > 0 && n % heads) || gate_splits < 0 ||
         gate_off < 0 || gate_off + n > gate_width || (dtype != 0 && dtype != 1))
         return EGPT_BAD_ARGUMENT;
     if (n_tokens == 0) return EGPT_OK;
     hipStream_t s = static_cast<hipStream_t>(stream);
+    if (row_ss && (gate_splits < 1 || ss_splits < 1 || hidden <= 0)) return EGPT_BAD_ARGUMENT;
+    const RowFactor factor{row_ss, ss_splits, n_tokens, hidden, norm_eps};
     const size_t total = static_cast<size_t>(n_tokens) * n;
     const size_t stride = static_cast<size_t>(n_tokens) * gate_width;
     const unsigned blocks = static_cast<unsigned>((total + 255) / 256);
     if (dtype == 0)
         sigmoid_gate_kernel<float><<<blocks, 256, 0, s>>>(static_cast<const float*>(x), heads,
-                                                          view_of<float>(gate, gate_splits, stride), gate_width, gate_off,
+                                                          view_of<float>(gate, gate_splits, stride), factor, gate_width, gate_off,
                                                           static_cast<float*>(out), n_tokens, n);
     else
         sigmoid_gate_kernel<bf16_t><<<blocks, 256, 0, s>>>(static_cast<const bf16_t*>(x), heads,
-                                                           view_of<bf16_t>(gate, gate_splits, stride), gate_width,
+                                                           view_of<bf16_t>(gate, gate_splits, stride), factor, gate_width,
                                                            gate_off, static_cast<bf16_t*>(out), n_tokens, n);
     EGPT_CHECK_LAUNCH();
     return EGPT_OK;

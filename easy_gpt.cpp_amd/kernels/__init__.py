@@ -32,7 +32,10 @@ Methods of a backend (T tokens, B requests, R rows, act = bfloat16 or float32):
   argmax(logits f32[R,V], out i32[R])            lowest index among equal maxima
   sample(logits f32[R,V], temperature f32[R], top_k i32[R], top_p f32[R], uniform f32[R], out i32[R])
 
-  embed_rmsnorm(token_ids i32[T], table act[V,H], weight act[H], eps, out f32[T,H])
+  (head_norm_store, latent_prep and sigmoid_gate also take row_ss f32[S2,T], hidden, norm_eps: the product, float32
+   partial sums, then still lacks each row's factor 1/sqrt(sum_s row_ss[s] / hidden + norm_eps), as `product_normed`
+   leaves it)
+  embed_rmsnorm(token_ids i32[T], table act[V,H], weight act[H], eps, out f32[T,H] | fixed point)
         out = table[id] / sqrt(mean(table[id]^2) + eps) * weight: an embedding with its norm, as the residual stream
   head_norm_store(proj act[T,W]|f32[S,T,W], q_out act[T,nq*dk], q_weight act[dk]|None, k_weight act[dk]|None, eps,
                   norm_values, slots i32[T]|None, k_cache, v_cache, nq, nkv, dk, dv, page_size)
@@ -102,12 +105,13 @@ class KernelBackend:
 
         return (h.double() * (1.0 / 4294967296.0)).float() if h.dtype == torch.int64 else h
 
-    def heads_product(self, x, w):
-        """x[h] w[h] for every head h: x act [heads, T, K] (any strides), w act [heads, K, N] -> act [heads, T, N].
-        The library's batched product (float32 operands are multiplied in float32)."""
+    def heads_product(self, x, w, out=None):
+        """x[h] w[h] for every head h: x act [heads, T, K] (any strides), w act [heads, K, N] -> act [heads, T, N]
+        (written into `out`, a view of those sizes whose rows are contiguous, if given).  The library's batched
+        product (float32 operands are multiplied in float32)."""
         import torch
 
-        return torch.bmm(x, w)
+        return torch.bmm(x, w) if out is None else torch.bmm(x, w, out=out)
 
     def product(self, x, w, unrounded=False, residual=None):
         """x w^T as act [m, n], or as float32 partial sums [splits, m, n] for a consumer that adds them up; or, given

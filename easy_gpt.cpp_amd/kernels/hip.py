@@ -28,7 +28,7 @@ def _load_library() -> ctypes.CDLL:
         lib = ctypes.CDLL(path)
     except (build.BuildError, OSError) as e:
         raise KernelsUnavailable(f"the HIP kernel library could not be built or loaded: {e}") from e
-    if lib.egpt_abi_version() != 18:
+    if lib.egpt_abi_version() != 19:
         raise KernelsUnavailable(f"{path} has an unexpected ABI version")
     return lib
 
@@ -101,10 +101,10 @@ class HipKernels(KernelBackend):
             "egpt_sample": [vp, vp, vp, vp, vp, vp, vp, i, i, vp],
             "egpt_sample_wide": [vp, vp, vp, vp, vp, vp, vp, i, i, vp],
             "egpt_gemm_gate_up_swiglu": [vp, vp, vp, i, i, i, i, vp],
-            "egpt_embed_rmsnorm": [vp, vp, vp, f, vp, i, i, i, i, vp],
-            "egpt_head_norm_store": [vp, i, vp, vp, vp, f, i, vp, vp, vp, i, i, i, i, i, i, i, vp],
-            "egpt_latent_prep": [vp, i, i, vp, vp, vp, f, vp, f, i, vp, vp, vp, i, i, i, i, i, i, i, vp],
-            "egpt_sigmoid_gate": [vp, i, vp, i, i, i, vp, i, i, i, vp],
+            "egpt_embed_rmsnorm": [vp, vp, vp, f, vp, i, i, i, i, i, vp],
+            "egpt_head_norm_store": [vp, i, vp, i, i, f, vp, vp, vp, f, i, vp, vp, vp, i, i, i, i, i, i, i, vp],
+            "egpt_latent_prep": [vp, i, vp, i, i, f, i, vp, vp, vp, f, vp, f, i, vp, vp, vp, i, i, i, i, i, i, i, vp],
+            "egpt_sigmoid_gate": [vp, i, vp, i, vp, i, i, f, i, i, vp, i, i, i, vp],
             "egpt_window_attention": [vp, vp, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, i, f, i, i, vp, i, vp],
             "egpt_window_attention_tiled": [vp, vp, vp, vp, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, i, f, i, i, vp, i, i,
                                             i, vp],
@@ -860,9 +860,18 @@ class HipKernels(KernelBackend):
         self._need(token_ids, "token_ids", _I32, (t,))
         self._need(table, "table")
         self._need(weight, "weight", table.dtype, (h,))
-        self._need(out, "out", _F32, (t, h))
+        self._need(out, "out", None, (t, h))
         self._run("egpt_embed_rmsnorm", token_ids.data_ptr(), table.data_ptr(), weight.data_ptr(), float(eps),
-                  out.data_ptr(), t, h, v, dt, self._stream())
+                  out.data_ptr(), self._fixed(out, "out"), t, h, v, dt, self._stream())
+
+    def _row_factor(self, row_ss, splits: int, t: int, hidden, eps):
+        """The arguments that say which factor the rows of a product still lack (none: a complete product)."""
+        if row_ss is None:
+            return None, 0, 0, 0.0
+        if splits < 1:
+            raise ValueError("a pending row factor needs float32 partial sums")
+        self._need(row_ss, "row_ss", _F32, (row_ss.shape[0], t))
+        return row_ss.data_ptr(), int(row_ss.shape[0]), int(hidden), float(eps)
 
     def _key_value_pages(self, k_cache, v_cache, dtype, nkv: int, page_size: int, dk: int, dv: int) -> None:
         self._need(k_cache, "k_cache", dtype)
@@ -875,7 +884,7 @@ class HipKernels(KernelBackend):
             raise ValueError("k_cache and v_cache must have the same number of pages")
 
     def head_norm_store(self, proj, q_out, q_weight, k_weight, eps, norm_values, slots, k_cache, v_cache, nq, nkv, dk, dv,
-                        page_size):
+                        page_size, row_ss=None, hidden=0, norm_eps=0.0):
         t = proj.shape[-2]
         dt = self._act(q_out, "q_out")
         splits = self._product(proj, "proj", q_out.dtype, t, (nq + nkv) * dk + nkv * dv)
@@ -886,13 +895,14 @@ class HipKernels(KernelBackend):
         if slots is not None:
             self._need(slots, "slots", _I32, (t,))
             self._key_value_pages(k_cache, v_cache, q_out.dtype, nkv, page_size, dk, dv)
-        self._run("egpt_head_norm_store", proj.data_ptr(), splits, q_out.data_ptr(), self._ptr(q_weight),
+        self._run("egpt_head_norm_store", proj.data_ptr(), splits, *self._row_factor(row_ss, splits, t, hidden, norm_eps),
+                  q_out.data_ptr(), self._ptr(q_weight),
                   self._ptr(k_weight), float(eps), 1 if norm_values else 0, self._ptr(slots),
                   self._ptr(k_cache) if slots is not None else None, self._ptr(v_cache) if slots is not None else None,
                   t, nq, nkv, dk, dv, page_size, dt, self._stream())
 
     def latent_prep(self, proj, q_plain, q_full, c_weight, eps, cos_sin, magnitude, rotary_dim, slots, k_cache, v_cache,
-                    nq, dim, rot, rank, page_size):
+                    nq, dim, rot, rank, page_size, row_ss=None, hidden=0, norm_eps=0.0):
         t, width = proj.shape[-2], proj.shape[-1]
         dt = self._act(q_full, "q_full")
         if width < nq * (dim + rot) + rank + rot:
@@ -909,16 +919,17 @@ class HipKernels(KernelBackend):
         if slots is not None:
             self._need(slots, "slots", _I32, (t,))
             self._key_value_pages(k_cache, v_cache, q_full.dtype, 1, page_size, rank + rot, rank)
-        self._run("egpt_latent_prep", proj.data_ptr(), splits, int(width), q_plain.data_ptr(), q_full.data_ptr(),
+        self._run("egpt_latent_prep", proj.data_ptr(), splits, *self._row_factor(row_ss, splits, t, hidden, norm_eps),
+                  int(width), q_plain.data_ptr(), q_full.data_ptr(),
                   c_weight.data_ptr(), float(eps), self._ptr(cos_sin) if rotary_dim else None, float(magnitude),
                   int(rotary_dim), self._ptr(slots), self._ptr(k_cache) if slots is not None else None,
                   self._ptr(v_cache) if slots is not None else None, t, nq, dim, rot, rank, page_size, dt, self._stream())
 
-    def heads_product(self, x, w):
+    def heads_product(self, x, w, out=None):
         with _FirstChoice():
-            return torch.bmm(x, w)
+            return torch.bmm(x, w) if out is None else torch.bmm(x, w, out=out)
 
-    def sigmoid_gate(self, x, heads, gate, gate_offset, out):
+    def sigmoid_gate(self, x, heads, gate, gate_offset, out, row_ss=None, hidden=0, norm_eps=0.0):
         t, n = out.shape
         dt = self._act(out, "out")
         self._need(out, "out")
@@ -927,7 +938,8 @@ class HipKernels(KernelBackend):
         splits = self._product(gate, "gate", out.dtype, t, width)
         if gate_offset < 0 or gate_offset + n > width:
             raise ValueError(f"gate columns {gate_offset}..{gate_offset + n} lie outside rows of {width} values")
-        self._run("egpt_sigmoid_gate", x.data_ptr(), int(heads), gate.data_ptr(), splits, int(width), int(gate_offset),
+        self._run("egpt_sigmoid_gate", x.data_ptr(), int(heads), gate.data_ptr(), splits,
+                  *self._row_factor(row_ss, splits, t, hidden, norm_eps), int(width), int(gate_offset),
                   out.data_ptr(), t, n, dt, self._stream())
 
     def window_attention(self, q, out, k_cache, v_cache, block_table, q_start, q_len, kv_len, nq, nkv, dk, dv, page_size,

@@ -45,8 +45,8 @@ class TokenEmbedding(Embedding):
 
 class NormedTokenEmbedding(TokenEmbedding):
     """x[t, :] = N(E[id_t, :]) with an RMS norm that has one gain for all coordinates (the tensor `prefix + norm_name`):
-    gather, statistics and the product with the gain in one kernel, in float32, written as the residual stream.  The
-    stream of such a model is float32 in steps of any size."""
+    gather, statistics and the product with the gain in one kernel, in float32, written as the residual stream (of the
+    kind that the backend names for the step's size)."""
 
     def __init__(self, prefix: str, hidden_size: int, vocab_size: int, eps: float, name: str = "weight",
                  norm_name: str = "norm"):
@@ -64,9 +64,11 @@ class NormedTokenEmbedding(TokenEmbedding):
         self.gain = gain.expand(self.hidden_size).to(device).contiguous()
 
     def forward(self, ctx) -> torch.Tensor:
+        k = kernels.backend()
         token_ids = ctx.token_ids
-        out = torch.empty((token_ids.shape[0], self.hidden_size), device=token_ids.device, dtype=torch.float32)
-        kernels.backend().embed_rmsnorm(token_ids, self.table, self.gain, self.eps, out)
+        out = torch.empty((token_ids.shape[0], self.hidden_size), device=token_ids.device,
+                          dtype=k.residual_dtype(token_ids.shape[0], self.table.dtype))
+        k.embed_rmsnorm(token_ids, self.table, self.gain, self.eps, out)
         return out
 
 

@@ -21,7 +21,7 @@ from __future__ import annotations
 import torch
 
 from .. import kernels
-from .base import CacheNeed, Mixer, PagedTensor, make_part, register_part
+from .base import CacheNeed, Mixer, PagedTensor, PendingNorm, make_part, register_part
 from .spec import ParamSpec, PartSpec
 
 
@@ -29,7 +29,49 @@ def _window(window) -> int | None:
     return int(window) if window else None
 
 
-class NormedAttention(Mixer):
+class _Projected:
+    """What a mixer's first phase leaves for its second: the input product, the factor its rows may still lack (a norm
+    that was folded into the product), and the stream that the output product may add itself into."""
+
+    __slots__ = ("proj", "factor", "residual", "t", "dtype", "device")
+
+    def __init__(self, proj, factor, residual, t, dtype, device):
+        self.proj, self.factor, self.residual, self.t, self.dtype, self.device = proj, factor, residual, t, dtype, device
+
+
+def _input_product(x, w, hidden_size) -> _Projected:
+    """x w^T for a mixer's input: from a tensor, or from a pending norm, which is folded into the product where the
+    backend has that kernel (the rows' 1/rms factor then goes on to the preparation kernel)."""
+    k = kernels.backend()
+    if isinstance(x, PendingNorm):
+        rms = x.rms()
+        fused = k.product_normed(x.h, x.delta, rms[0], w) if rms is not None else None
+        if fused is not None:
+            proj, row_ss, h_new = fused
+            x.applied(h_new)
+            return _Projected(proj, dict(row_ss=row_ss, hidden=hidden_size, norm_eps=rms[1]), x.residual(), h_new.shape[0],
+                              w.dtype, h_new.device)
+        pending, x = x, x.materialize()
+        return _Projected(k.product(x, w, unrounded=True), {}, pending.residual(), x.shape[0], x.dtype, x.device)
+    return _Projected(k.product(x, w, unrounded=True), {}, None, x.shape[0], x.dtype, x.device)
+
+
+def _output_product(heads_out, w, residual):
+    out = kernels.backend().product(heads_out, w, unrounded=True, residual=residual)
+    return None if out is residual and residual is not None else out
+
+
+class _TwoPhases(Mixer):
+    """forward = finish(project(x)): `project` is all that reads the mixer's input (and, through a pending norm, the
+    residual stream); `finish` is the rest, and may add the output into the stream."""
+
+    takes_pending_norm = True
+
+    def forward(self, x, ctx, cache, state=None):
+        return self.finish(self.project(x, ctx), ctx, cache, state)
+
+
+class NormedAttention(_TwoPhases):
     graph_safe = True
 
     def __init__(self, prefix: str, hidden_size: int, n_heads: int, n_kv_heads: int, key_dim: int, value_dim: int,
@@ -78,22 +120,24 @@ class NormedAttention(Mixer):
             self.q_weight = self._to(get(p + n["q_norm"]), "compute", dtype, device)
             self.k_weight = self._to(get(p + n["k_norm"]), "compute", dtype, device)
 
-    def forward(self, x, ctx, cache, state=None):
+    def project(self, x, ctx):
+        return _input_product(x, self.w_qkv, self.hidden_size)
+
+    def finish(self, p, ctx, cache, state=None):
         k = kernels.backend()
-        t = x.shape[0]
-        proj = k.product(x, self.w_qkv, unrounded=True)
-        q = torch.empty((t, self.n_heads * self.key_dim), dtype=x.dtype, device=x.device)
-        k.head_norm_store(proj, q, self.q_weight, self.k_weight, self.eps, self.norm_values,
+        t = p.t
+        q = torch.empty((t, self.n_heads * self.key_dim), dtype=p.dtype, device=p.device)
+        k.head_norm_store(p.proj, q, self.q_weight, self.k_weight, self.eps, self.norm_values,
                           cache.slots if cache.writes else None, cache.k, cache.v, self.n_heads, self.n_kv_heads,
-                          self.key_dim, self.value_dim, cache.page_size)
-        attn = torch.empty((t, self.n_heads * self.value_dim), dtype=x.dtype, device=x.device)
+                          self.key_dim, self.value_dim, cache.page_size, **p.factor)
+        attn = torch.empty((t, self.n_heads * self.value_dim), dtype=p.dtype, device=p.device)
         k.window_attention(q, attn, cache.k, cache.v, cache.block_table, ctx.q_start, ctx.q_len, ctx.kv_len,
                            self.n_heads, self.n_kv_heads, self.key_dim, self.value_dim, cache.page_size, self.scale,
                            self.window or 0, self.keep_first, None, ctx.max_q_len, ctx.max_kv_len)
-        return k.product(attn, self.w_o, unrounded=True)
+        return _output_product(attn, self.w_o, p.residual)
 
 
-class LatentAttention(Mixer):
+class LatentAttention(_TwoPhases):
     graph_safe = True
 
     def __init__(self, prefix: str, hidden_size: int, n_heads: int, plain_dim: int, rotated_dim: int, value_dim: int,
@@ -157,31 +201,34 @@ class LatentAttention(Mixer):
             self.sink = get(p + n["sink"]).to(torch.float32).to(device).contiguous()
         self.position.load(get, dtype, device)
 
-    def forward(self, x, ctx, cache, state=None):
+    def project(self, x, ctx):
+        return _input_product(x, self.w_in, self.hidden_size)
+
+    def finish(self, p, ctx, cache, state=None):
         k = kernels.backend()
-        t, nh, rank, rot = x.shape[0], self.n_heads, self.latent_dim, self.rotated_dim
-        proj = k.product(x, self.w_in, unrounded=True)
-        q_plain = torch.empty((t, nh, self.plain_dim), dtype=x.dtype, device=x.device)
-        q_full = torch.empty((t, nh, rank + rot), dtype=x.dtype, device=x.device)
-        rotary = self.position.rotary(x.device)
+        t, nh, rank, rot = p.t, self.n_heads, self.latent_dim, self.rotated_dim
+        q_plain = torch.empty((t, nh, self.plain_dim), dtype=p.dtype, device=p.device)
+        q_full = torch.empty((t, nh, rank + rot), dtype=p.dtype, device=p.device)
+        rotary = self.position.rotary(p.device)
         cos_sin = self.position.table(ctx) if rotary is not None else None
-        k.latent_prep(proj, q_plain, q_full, self.c_weight, self.eps, cos_sin, getattr(self.position, "magnitude", 1.0),
+        k.latent_prep(p.proj, q_plain, q_full, self.c_weight, self.eps, cos_sin, getattr(self.position, "magnitude", 1.0),
                       rotary[1] if rotary is not None else 0, cache.slots if cache.writes else None, cache.k, cache.v,
-                      nh, self.plain_dim, rot, rank, cache.page_size)
-        # the queries' unrotated parts carried into the latent space, head by head
-        q_full[:, :, :rank].copy_(k.heads_product(q_plain.transpose(0, 1), self.w_up_k).transpose(0, 1))
-        o_latent = torch.empty((t, nh * rank), dtype=x.dtype, device=x.device)
+                      nh, self.plain_dim, rot, rank, cache.page_size, **p.factor)
+        # the queries' unrotated parts carried into the latent space, head by head, into their places before the
+        # rotated parts
+        k.heads_product(q_plain.transpose(0, 1), self.w_up_k, out=q_full[:, :, :rank].transpose(0, 1))
+        o_latent = torch.empty((t, nh * rank), dtype=p.dtype, device=p.device)
         k.window_attention(q_full.view(t, nh * (rank + rot)), o_latent, cache.k, cache.v, cache.block_table, ctx.q_start,
                            ctx.q_len, ctx.kv_len, nh, 1, rank + rot, rank, cache.page_size, self.scale, self.window or 0,
                            0, self.sink, ctx.max_q_len, ctx.max_kv_len)
         # and the heads' outputs carried back: [heads, T, value]
         o = k.heads_product(o_latent.view(t, nh, rank).transpose(0, 1), self.w_up_v)
         if self.gated:
-            heads_out = torch.empty((t, self.out_width), dtype=x.dtype, device=x.device)
-            k.sigmoid_gate(o, nh, proj, self.q_width + self.down_width, heads_out)
+            heads_out = torch.empty((t, self.out_width), dtype=p.dtype, device=p.device)
+            k.sigmoid_gate(o, nh, p.proj, self.q_width + self.down_width, heads_out, **p.factor)
         else:
             heads_out = o.transpose(0, 1).reshape(t, self.out_width)
-        return k.product(heads_out, self.w_o, unrounded=True)
+        return _output_product(heads_out, self.w_o, p.residual)
 
 
 register_part("mixer", "normed_attention", NormedAttention)

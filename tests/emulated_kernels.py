@@ -161,8 +161,12 @@ class EmulatedKernels(KernelBackend):
             keys = torch.cat([c, turn(shared)], dim=-1).view(t, 1, rank + rot)
             self._store(k_cache, v_cache, slots, page_size, keys, c.view(t, 1, rank))
 
-    def heads_product(self, x, w):
-        return torch.bmm(x.to(F64), w.to(F64)).to(x.dtype)
+    def heads_product(self, x, w, out=None):
+        y = torch.bmm(x.to(F64), w.to(F64)).to(x.dtype)
+        if out is None:
+            return y
+        out.copy_(y)
+        return out
 
     def sigmoid_gate(self, x, heads, gate, gate_offset, out):
         t, n = out.shape
