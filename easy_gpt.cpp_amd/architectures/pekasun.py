@@ -32,7 +32,7 @@ def _mixer_spec(layer: LayerConfig, prefix: str, eps: float) -> PartSpec:
     return PartSpec(
         "latent_attention",
         dict(n_heads=m.heads, plain_dim=m.dim, rotated_dim=m.rot_dim, value_dim=m.vdim, latent_dim=m.kv_rank, scale=m.scale,
-             window=m.window, eps=eps, sink=True, gated=True, position=position,
+             window=m.window, keep_first=m.keep_first, eps=eps, sink=True, gated=True, position=position,
              names=dict(q="q", down="dkv", down_norm="dkv.norm", up_k="uk", up_v="uv", sink="sink", gate="g", o="o")),
         prefix=prefix,
     )

@@ -46,7 +46,7 @@ class RotationConfig:
 @dataclass(frozen=True)
 class MixerConfig:
     """Sizes and constants of one mixer.  kind 'attention': heads, kv_heads, dim, vdim, scale, window, keep_first.
-    kind 'latent_attention': heads, dim, rot_dim, vdim, kv_rank, scale, window, rotation."""
+    kind 'latent_attention': heads, dim, rot_dim, vdim, kv_rank, scale, window, keep_first, rotation."""
 
     kind: str
     heads: int
@@ -90,9 +90,7 @@ class MixerConfig:
                 rotation = RotationConfig.from_dict(data["rot"], where + ".rot")
                 if rotation.dims > rot_dim:
                     raise ConfigError(f"{where}: rot.dims ({rotation.dims}) is larger than rot_dim ({rot_dim})")
-            if keep_first:
-                raise ConfigError(f"{where}: the latent attention's window keeps no first tokens ('mask.keep_first')")
-            return cls(kind, heads, dim, vdim, scale, window, 0, rot_dim=rot_dim, kv_rank=rank, rotation=rotation)
+            return cls(kind, heads, dim, vdim, scale, window, keep_first, rot_dim=rot_dim, kv_rank=rank, rotation=rotation)
         raise ConfigError(f"{where}: unknown layer type '{kind}' (known: attention, latent_attention)")
 
 

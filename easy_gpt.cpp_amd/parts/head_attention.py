@@ -142,7 +142,7 @@ class LatentAttention(_TwoPhases):
 
     def __init__(self, prefix: str, hidden_size: int, n_heads: int, plain_dim: int, rotated_dim: int, value_dim: int,
                  latent_dim: int, scale: float, eps: float, position: PartSpec, window: int | None = None,
-                 sink: bool = False, gated: bool = False, names: dict | None = None):
+                 keep_first: int = 0, sink: bool = False, gated: bool = False, names: dict | None = None):
         """plain_dim / rotated_dim: a head's unrotated and rotated query/key places (a query head is laid out
         [plain | rotated]); latent_dim: the width of the cached latent.  names: tensor names behind `prefix` of q, down
         (rows: latent, then the shared rotated key), down_norm, up_k, up_v, sink, gate, o."""
@@ -156,6 +156,7 @@ class LatentAttention(_TwoPhases):
         self.value_dim, self.latent_dim = int(value_dim), int(latent_dim)
         self.scale, self.eps = float(scale), float(eps)
         self.window = _window(window)
+        self.keep_first = int(keep_first) if self.window else 0
         self.has_sink, self.gated = bool(sink), bool(gated)
         self.position = make_part("position_encoding", position, head_dim=max(self.rotated_dim, 2))
         self.names = dict(q="q", down="down", down_norm="down_norm", up_k="up_k", up_v="up_v", sink="sink", gate="gate", o="o")
@@ -168,7 +169,7 @@ class LatentAttention(_TwoPhases):
     def cache_need(self):
         # one key/value head: keys [latent | rotated part], values the latent, transposed within a page
         return CacheNeed((PagedTensor("k", (1, self.latent_dim + self.rotated_dim), 1),
-                          PagedTensor("v", (1, self.latent_dim), 2)), self.window)
+                          PagedTensor("v", (1, self.latent_dim), 2)), self.window, self.keep_first)
 
     def param_specs(self):
         p, h, n = self.prefix, self.hidden_size, self.names
@@ -220,7 +221,7 @@ class LatentAttention(_TwoPhases):
         o_latent = torch.empty((t, nh * rank), dtype=p.dtype, device=p.device)
         k.window_attention(q_full.view(t, nh * (rank + rot)), o_latent, cache.k, cache.v, cache.block_table, ctx.q_start,
                            ctx.q_len, ctx.kv_len, nh, 1, rank + rot, rank, cache.page_size, self.scale, self.window or 0,
-                           0, self.sink, ctx.max_q_len, ctx.max_kv_len)
+                           self.keep_first, self.sink, ctx.max_q_len, ctx.max_kv_len)
         # and the heads' outputs carried back: [heads, T, value]
         o = k.heads_product(o_latent.view(t, nh, rank).transpose(0, 1), self.w_up_v)
         if self.gated:

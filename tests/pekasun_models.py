@@ -12,13 +12,13 @@ import torch
 from easy_gpt.cpp_amd.weights import write_safetensors
 
 
-def latent(heads, dim, rot_dim, vdim, rank, window, scale, base=10000.0, dims=None, scaling=None):
+def latent(heads, dim, rot_dim, vdim, rank, window, scale, base=10000.0, dims=None, scaling=None, keep_first=None):
     rot = None if rot_dim == 0 else {"base": base, "dims": rot_dim if dims is None else dims, "scaling": scaling}
     if rot is not None and scaling is None:
         del rot["scaling"]
     m = {"heads": heads, "dim": dim, "rot_dim": rot_dim, "vdim": vdim, "kv_rank": rank, "scale": scale, "rot": rot}
     if window:
-        m["mask"] = {"size": window}
+        m["mask"] = {"size": window} if keep_first is None else {"size": window, "keep_first": keep_first}
     return {"type": "latent_attention", "mixer": m}
 
 
@@ -71,7 +71,17 @@ CONFIG_C = {
         layer(latent(4, 32, 16, 32, 48, 16, 0.15, base=20000.0), 160, weights_of=0),
     ],
 }
-CONFIGS = {"A": (CONFIG_A, 5), "B": (CONFIG_B, 6), "C": (CONFIG_C, 7)}
+# sizes that are multiples of nothing: a width of 100, heads of 12 and 20, a latent of 36 with an odd rotated part of 7
+# (six places rotated), an inner width of 50, a latent window that keeps two tokens
+CONFIG_E = {
+    "architecture": "Pekasun", "vocab": 333, "width": 100, "norm": {"eps": 1e-6},
+    "layers": [
+        layer(latent(3, 12, 7, 20, 36, 9, 0.3, base=3000.0, dims=6, keep_first=2), 50),
+        layer(attention(3, 1, 12, 20, 11, 2, 0.35), 50),
+        layer(attention(5, 5, 20, 12, 6, 0, -0.3), None),
+    ],
+}
+CONFIGS = {"A": (CONFIG_A, 5), "B": (CONFIG_B, 6), "C": (CONFIG_C, 7), "E": (CONFIG_E, 9)}
 
 
 def draw_weights(cfg: dict, seed: int, sharp: float = 3.0) -> dict[str, torch.Tensor]:

@@ -161,15 +161,15 @@ def latent_attention(h, w, p, m, eps):
     dkv = h @ w[p + "dkv"].T
     c = vector_norm(dkv[:, :rank], w[p + "dkv.norm"], eps)
     k_rot = dkv[:, rank:]
-    freqs, mag = yarn_frequencies(m["rot"])
+    freqs, mag = yarn_frequencies(m["rot"]) if m.get("rot") else (torch.zeros(0, dtype=F64), 1.0)
     q_un, q_rot = q[..., :d], q[..., d:]
     q_rot = rotate_interleaved(q_rot.transpose(0, 1), pos, freqs, mag).transpose(0, 1)
     k_rot = rotate_interleaved(k_rot, pos, freqs, mag)
     k_un = (c @ w[p + "uk"].T).reshape(n, H, d)
     v = (c @ w[p + "uv"].T).reshape(n, H, dv)
     scores = (torch.einsum("ihd,jhd->hij", q_un, k_un) + torch.einsum("ihd,jd->hij", q_rot, k_rot)) * float(m["scale"])
-    size = int((m.get("mask") or {}).get("size", 1 << 60))
-    vis = visible_window_keep_first(n, size, 0)
+    mask = m.get("mask") or {}
+    vis = visible_window_keep_first(n, int(mask.get("size", 1 << 60)), int(mask.get("keep_first", 0)))
     pr = softmax_with_sink(scores, vis, w[p + "sink"])
     o = torch.einsum("hij,jhd->ihd", pr, v).reshape(n, H * dv)
     o = o * torch.sigmoid(h @ w[p + "g"].T)

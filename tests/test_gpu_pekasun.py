@@ -60,7 +60,7 @@ def plain_rows(model_dir, reqs):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D", "E"])
 def test_every_cutting_agrees_with_plain(models, name, dtype):
     cfg = ALL[name][0]
     reqs = H.make_requests(cfg["vocab"], [150, 1, 47, 2, 96], seed=21)
@@ -113,6 +113,19 @@ def test_long_decoding_passes_every_window_and_gives_pages_back(models, name, dt
     windowed = [g for g, need in enumerate(eng.cache.groups) if need.window is not None and need.window < 100]
     tables = eng.cache.requests["again"].tables
     assert windowed and all(sum(p >= 0 for p in tables[g]) < len(tables[g]) for g in windowed)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_prompt_longer_than_any_graph_in_one_step(models, dtype):
+    """2,600 tokens in one step (steps beyond 2,048 tokens run kernel by kernel), then tokens one by one."""
+    name = "D"
+    cfg = ALL[name][0]
+    reqs = H.make_requests(cfg["vocab"], [2610], seed=88)
+    ref = plain_rows(models[name], reqs)
+    eng = engine(models[name], dtype, page_size=16, max_tokens=2624, max_requests=1)
+    rows = H.replay(eng, H.trace_last_decoded(reqs, 10))
+    assert len(rows) == 2610
+    H.assert_rows_match(rows, ref, TOL[dtype], f"long prompt {dtype}")
 
 
 def test_a_batch_gives_each_request_what_it_gets_alone(models):
