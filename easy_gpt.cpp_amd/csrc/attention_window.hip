@@ -219,11 +219,19 @@ struct WindowArgs {
     const int32_t* kv_len;
     const float* sink;
     int table_width, n_seqs, n_tokens, nq, nkv, dk, dv, page_size, window, keep_first, n_splits;
+    int page_shift;          // log2 of the page size if that is a power of two, else -1
     float scale;
 };
 
+__device__ __forceinline__ int page_index(int key, int page_size, int page_shift) {
+    return page_shift >= 0 ? key >> page_shift : key / page_size;
+}
+__device__ __forceinline__ int place_in_page(int key, int page_size, int page_shift) {
+    return page_shift >= 0 ? key & (page_size - 1) : key % page_size;
+}
+
 template <typename T, int DT, int RT, int RW>
-__global__ __launch_bounds__(64 * RT) void window_attention_tiled_kernel(WindowArgs a) {
+__global__ __launch_bounds__(64 * RT, (DT * RW <= 8 ? 2 : 1)) void window_attention_tiled_kernel(WindowArgs a) {
     constexpr int E = 16 / sizeof(T);             // elements in 16 bytes
     constexpr int KT = sizeof(T) == 2 ? 64 : 32;  // keys per chunk
     constexpr int NKT = KT / 16;                  // tiles of 16 keys in a chunk
@@ -239,6 +247,7 @@ __global__ __launch_bounds__(64 * RT) void window_attention_tiled_kernel(WindowA
     const T* __restrict__ k_cache = static_cast<const T*>(a.k_cache);
     const T* __restrict__ v_cache = static_cast<const T*>(a.v_cache);
     const int dk = a.dk, dv = a.dv, nq = a.nq, nkv = a.nkv, page_size = a.page_size, window = a.window;
+    const int page_shift = a.page_shift;
     const int n_pieces = (dk + PF - 1) / PF;
     const int krow = n_pieces * PF + E;           // padded LDS row of keys and of queries
     const int k_pieces = dk / E;                  // 16-byte pieces of a key
@@ -338,32 +347,48 @@ __global__ __launch_bounds__(64 * RT) void window_attention_tiled_kernel(WindowA
     constexpr int VKP = KT / E;   // 16-byte pieces of a value row
     w_u32x4 k_regs[KU], v_regs[VU];
     const int k_total = KT * k_pieces, v_total = dv * VKP;
-    auto fetch = [&](int c) {
+    // which key of a chunk and which piece of it this thread's loads take (the same in every chunk)
+    int k_row[KU], k_col[KU];
+#pragma unroll
+    for (int u = 0; u < KU; ++u) {
+        const int idx = tid + u * THREADS;
+        k_row[u] = idx < k_total ? idx / k_pieces : -1;
+        k_col[u] = idx < k_total ? idx % k_pieces : 0;
+    }
+    // page numbers are looked up a chunk ahead of the loads that need them, so that an iteration waits for one trip
+    // to memory, not for two that depend on each other
+    int k_page[KU], v_page[VU];
+    auto lookup = [&](int c) {
         const bool any = c < c_end;
         const int tile = c < kept_chunks ? c : t_begin + (c - kept_chunks);
         const int key0 = tile * KT;
-        long k_page[KU], v_page[VU];
 #pragma unroll
         for (int u = 0; u < KU; ++u) {
-            const int idx = tid + u * THREADS;
-            const int j = key0 + idx / k_pieces;
+            const int j = key0 + k_row[u];
             k_page[u] = -1;
-            if (any && idx < k_total && j <= p_max && (j >= lo_blk || j < keep)) k_page[u] = table[j / page_size];
+            if (any && k_row[u] >= 0 && j <= p_max && (j >= lo_blk || j < keep))
+                k_page[u] = table[page_index(j, page_size, page_shift)];
         }
 #pragma unroll
         for (int u = 0; u < VU; ++u) {
             const int idx = tid + u * THREADS;
             const int j = key0 + (idx % VKP) * E;
             v_page[u] = -1;
-            if (any && idx < v_total && j <= p_max && (j + E - 1 >= lo_blk || j < keep)) v_page[u] = table[j / page_size];
+            if (any && idx < v_total && j <= p_max && (j + E - 1 >= lo_blk || j < keep))
+                v_page[u] = table[page_index(j, page_size, page_shift)];
         }
+    };
+    auto fetch = [&](int c) {
+        const int tile = c < kept_chunks ? c : t_begin + (c - kept_chunks);
+        const int key0 = tile * KT;
 #pragma unroll
         for (int u = 0; u < KU; ++u) {
-            const int idx = tid + u * THREADS;
-            const int j = key0 + idx / k_pieces, cc = idx % k_pieces;
+            const int j = key0 + k_row[u];
             k_regs[u] = w_u32x4{0u, 0u, 0u, 0u};
             if (k_page[u] >= 0)
-                k_regs[u] = *reinterpret_cast<const w_u32x4*>(k_cache + ((k_page[u] * nkv + kh) * page_size + j % page_size) * dk + cc * E);
+                k_regs[u] = *reinterpret_cast<const w_u32x4*>(
+                    k_cache + ((static_cast<long>(k_page[u]) * nkv + kh) * page_size + place_in_page(j, page_size, page_shift)) * dk +
+                    k_col[u] * E);
         }
 #pragma unroll
         for (int u = 0; u < VU; ++u) {
@@ -371,7 +396,8 @@ __global__ __launch_bounds__(64 * RT) void window_attention_tiled_kernel(WindowA
             const int f = idx / VKP, j = key0 + (idx % VKP) * E;
             w_u32x4 v = w_u32x4{0u, 0u, 0u, 0u};
             if (v_page[u] >= 0) {
-                v = *reinterpret_cast<const w_u32x4*>(v_cache + ((v_page[u] * nkv + kh) * dv + f) * page_size + j % page_size);
+                v = *reinterpret_cast<const w_u32x4*>(
+                    v_cache + ((static_cast<long>(v_page[u]) * nkv + kh) * dv + f) * page_size + place_in_page(j, page_size, page_shift));
                 if (j + E > kv) {         // places of the page that no token has written yet may hold anything
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
@@ -389,10 +415,8 @@ __global__ __launch_bounds__(64 * RT) void window_attention_tiled_kernel(WindowA
     };
     auto stash = [&]() {
 #pragma unroll
-        for (int u = 0; u < KU; ++u) {
-            const int idx = tid + u * THREADS;
-            if (idx < k_total) *reinterpret_cast<w_u32x4*>(k_s + (idx / k_pieces) * krow + (idx % k_pieces) * E) = k_regs[u];
-        }
+        for (int u = 0; u < KU; ++u)
+            if (k_row[u] >= 0) *reinterpret_cast<w_u32x4*>(k_s + k_row[u] * krow + k_col[u] * E) = k_regs[u];
 #pragma unroll
         for (int u = 0; u < VU; ++u) {
             const int idx = tid + u * THREADS;
@@ -409,7 +433,9 @@ __global__ __launch_bounds__(64 * RT) void window_attention_tiled_kernel(WindowA
         }
     };
 
+    lookup(c_begin);
     fetch(c_begin);
+    lookup(c_begin + 1);
     for (int c = c_begin; c < c_end; ++c) {
         const int tile = c < kept_chunks ? c : t_begin + (c - kept_chunks);
         const int key0 = tile * KT;
@@ -417,6 +443,7 @@ __global__ __launch_bounds__(64 * RT) void window_attention_tiled_kernel(WindowA
         stash();
         __syncthreads();
         fetch(c + 1);                     // in flight while this chunk is computed; behind the last chunk nothing is read
+        lookup(c + 2);
         if (!wave_active) continue;
         // ---- scores of this wavefront's rows against the chunk's keys: a key operand serves all of its row tiles
         w_f32x4 acc[RW][NKT];
@@ -661,6 +688,9 @@ extern "C" int egpt_window_attention_tiled(const void* q, void* out, float* part
     a.block_table = block_table; a.q_start = q_start; a.q_len = q_len; a.kv_len = kv_len; a.sink = sink;
     a.table_width = table_width; a.n_seqs = n_seqs; a.n_tokens = n_tokens; a.nq = nq; a.nkv = nkv; a.dk = dk; a.dv = dv;
     a.page_size = page_size; a.window = window; a.keep_first = keep_first; a.n_splits = n_splits; a.scale = scale;
+    a.page_shift = -1;
+    for (int sh = 0; sh < 30; ++sh)
+        if ((1 << sh) == page_size) a.page_shift = sh;
     int code;
     if (dtype == 0)
         code = launch_tiled_for_dv<float>(a, n_tokens, row_tiles, s);

@@ -1002,12 +1002,13 @@ class HipKernels(KernelBackend):
             row_tiles = 4
         if lds(row_tiles) > 160 * 1024:
             return None
-        workgroups = (-(-t * group // (16 * row_tiles)) + b) * nkv
+        # workgroups that have rows (a request's rows start a workgroup of their own)
+        workgroups = min(b * -(-max_q_len * group // (16 * row_tiles)), -(-t * group // (16 * row_tiles)) + b) * nkv
         span = min(max_kv_len, window + min(max_q_len, 64) + chunk) if window else max_kv_len
         chunks = -(-span // chunk) + (-(-min(keep_first, max_kv_len) // chunk) if window else 0)
         n_splits = 1
-        if workgroups < 256 and chunks > 1:
-            n_splits = max(1, min(chunks, -(-512 // workgroups), 64))
+        if workgroups < 512 and chunks > 1:
+            n_splits = max(1, min(chunks, -(-1024 // workgroups), 64))
         return row_tiles, n_splits
 
     def swiglu(self, gate_up, out, row_ss=None, hidden=0, eps=0.0):

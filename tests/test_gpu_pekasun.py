@@ -196,3 +196,28 @@ def test_trace_run_as_a_subprocess(models, tmp_path, dtype):
     assert p.wait(timeout=60) == 0
     assert len(rows) > 60
     H.assert_rows_match(rows, ref, TOL[dtype], f"trace_run {dtype}")
+
+
+def test_the_command_line_generates_with_a_pekasun_folder(models, tmp_path):
+    """bin/easy_llm on a Pekasun folder, greedy in float32: the tokens are the plain model's (the weights of the tests
+    leave no near-ties), from a prompt on the command line and from a prompt file in portions of 16."""
+    name = "A"
+    prompt = [5, 17, 3, 250, 9, 44, 1]
+    cmd = [sys.executable, os.path.join(ROOT, "bin", "easy_llm"), "--model", models[name], "--dtype", "float32", "--greedy",
+           "--ignore-eos", "--max-new-tokens", "12"]
+    p = subprocess.run(cmd + [" ".join(map(str, prompt))], capture_output=True, text=True, timeout=110, cwd=ROOT)
+    assert p.returncode == 0, p.stderr[-2000:]
+    c, w = P.read_model(models[name])
+    out = [int(t) for t in p.stdout.split()]
+    assert len(out) == 12
+    logits = P.forward(c, w, prompt + out)
+    for i, tok in enumerate(out):
+        row = logits[len(prompt) + i - 1]
+        assert float(row.max() - row[tok]) <= 1e-4 * float(row.abs().max()), (i, tok)
+    (tmp_path / "prompts.txt").write_text("3 4 5\n" + " ".join(str(7 + i % 90) for i in range(50)) + "\n")
+    p = subprocess.run(cmd + ["-f", str(tmp_path / "prompts.txt"), "--prefill-chunk", "16", "--cache-tokens", "512"],
+                       capture_output=True, text=True, timeout=110, cwd=str(tmp_path),
+                       env=dict(os.environ, PYTHONPATH=ROOT + os.pathsep + os.environ.get("PYTHONPATH", "")))
+    assert p.returncode == 0, p.stderr[-2000:]
+    lines = (tmp_path / "prompts_output.txt").read_text().splitlines()
+    assert len(lines) == 2 and all(len(ln.split()) == 12 for ln in lines)
