@@ -297,6 +297,20 @@ __global__ __launch_bounds__(64 * RT, (DT * RW <= 8 ? 2 : 1)) void window_attent
         lo_row[w] = (window > 0 && valid[w]) ? max(0, p_row[w] - window + 1) : 0;
     }
 
+    // the smallest position and the largest window start among a tile's rows (rows of no token aside)
+    int tile_p_min[RW], tile_lo_max[RW];
+#pragma unroll
+    for (int w = 0; w < RW; ++w) {
+        int pm = valid[w] ? p_row[w] : 0x7fffffff, lm = valid[w] ? lo_row[w] : 0;
+#pragma unroll
+        for (int off = kWave / 2; off > 0; off >>= 1) {
+            pm = min(pm, __shfl_xor(pm, off, kWave));
+            lm = max(lm, __shfl_xor(lm, off, kWave));
+        }
+        tile_p_min[w] = pm == 0x7fffffff ? -1 : pm;
+        tile_lo_max[w] = lm;
+    }
+
     // queries into LDS, zeros beyond the key size and in rows that belong to no token; the pads of the key rows and the
     // value rows beyond the value size are zeroed once, the chunks never write there
     {
@@ -347,35 +361,51 @@ __global__ __launch_bounds__(64 * RT, (DT * RW <= 8 ? 2 : 1)) void window_attent
     constexpr int VKP = KT / E;   // 16-byte pieces of a value row
     w_u32x4 k_regs[KU], v_regs[VU];
     const int k_total = KT * k_pieces, v_total = dv * VKP;
-    // which key of a chunk and which piece of it this thread's loads take (the same in every chunk)
-    int k_row[KU], k_col[KU];
+    // which key of a chunk and which piece of it this thread's loads take, where they go in LDS and where they lie in a
+    // page's block (the same in every chunk); a thread has ku_n pieces of keys to take, the same for all threads but
+    // the last ones of the last round
+    const int ku_n = (k_total + THREADS - 1) / THREADS;
+    int k_row[KU], k_lds[KU], k_off[KU];
 #pragma unroll
     for (int u = 0; u < KU; ++u) {
         const int idx = tid + u * THREADS;
-        k_row[u] = idx < k_total ? idx / k_pieces : -1;
-        k_col[u] = idx < k_total ? idx % k_pieces : 0;
+        const bool used = idx < k_total;
+        k_row[u] = used ? idx / k_pieces : -(1 << 28);          // (a key no chunk holds)
+        k_lds[u] = used ? (idx / k_pieces) * krow + (idx % k_pieces) * E : 0;
+        k_off[u] = kh * page_size * dk + (used ? (idx % k_pieces) * E : 0);
     }
+    int v_key[VU], v_lds[VU];
+    long v_off[VU];
+#pragma unroll
+    for (int u = 0; u < VU; ++u) {
+        const int idx = tid + u * THREADS;
+        const bool used = idx < v_total;
+        const int f = idx / VKP, vk = (idx % VKP) * E;
+        v_key[u] = used ? vk : -(1 << 28);
+        v_off[u] = (static_cast<long>(kh) * dv + f) * page_size;
+        // where the E keys go: as they are (float32), or in the order in which a lane takes them (bfloat16: within 32
+        // keys by quarter of the wavefront, tile, key)
+        v_lds[u] = f * VROW + (sizeof(T) == 4 ? vk : (vk / 32) * 32 + ((vk % 16) / 4) * 8 + ((vk % 32) / 16) * 4);
+    }
+    const long k_page_stride = static_cast<long>(nkv) * page_size * dk, v_page_stride = static_cast<long>(nkv) * dv * page_size;
     // page numbers are looked up a chunk ahead of the loads that need them, so that an iteration waits for one trip
     // to memory, not for two that depend on each other
     int k_page[KU], v_page[VU];
     auto lookup = [&](int c) {
-        const bool any = c < c_end;
         const int tile = c < kept_chunks ? c : t_begin + (c - kept_chunks);
-        const int key0 = tile * KT;
+        const int key0 = c < c_end ? tile * KT : (1 << 29);        // behind the last chunk: keys that nobody sees
 #pragma unroll
         for (int u = 0; u < KU; ++u) {
+            if (u >= ku_n) break;
             const int j = key0 + k_row[u];
             k_page[u] = -1;
-            if (any && k_row[u] >= 0 && j <= p_max && (j >= lo_blk || j < keep))
-                k_page[u] = table[page_index(j, page_size, page_shift)];
+            if (j >= 0 && j <= p_max && (j >= lo_blk || j < keep)) k_page[u] = table[page_index(j, page_size, page_shift)];
         }
 #pragma unroll
         for (int u = 0; u < VU; ++u) {
-            const int idx = tid + u * THREADS;
-            const int j = key0 + (idx % VKP) * E;
+            const int j = key0 + v_key[u];
             v_page[u] = -1;
-            if (any && idx < v_total && j <= p_max && (j + E - 1 >= lo_blk || j < keep))
-                v_page[u] = table[page_index(j, page_size, page_shift)];
+            if (j >= 0 && j <= p_max && (j + E - 1 >= lo_blk || j < keep)) v_page[u] = table[page_index(j, page_size, page_shift)];
         }
     };
     auto fetch = [&](int c) {
@@ -383,21 +413,19 @@ __global__ __launch_bounds__(64 * RT, (DT * RW <= 8 ? 2 : 1)) void window_attent
         const int key0 = tile * KT;
 #pragma unroll
         for (int u = 0; u < KU; ++u) {
-            const int j = key0 + k_row[u];
+            if (u >= ku_n) break;
             k_regs[u] = w_u32x4{0u, 0u, 0u, 0u};
             if (k_page[u] >= 0)
                 k_regs[u] = *reinterpret_cast<const w_u32x4*>(
-                    k_cache + ((static_cast<long>(k_page[u]) * nkv + kh) * page_size + place_in_page(j, page_size, page_shift)) * dk +
-                    k_col[u] * E);
+                    k_cache + k_page[u] * k_page_stride + (place_in_page(key0 + k_row[u], page_size, page_shift) * dk + k_off[u]));
         }
 #pragma unroll
         for (int u = 0; u < VU; ++u) {
-            const int idx = tid + u * THREADS;
-            const int f = idx / VKP, j = key0 + (idx % VKP) * E;
+            const int j = key0 + v_key[u];
             w_u32x4 v = w_u32x4{0u, 0u, 0u, 0u};
             if (v_page[u] >= 0) {
                 v = *reinterpret_cast<const w_u32x4*>(
-                    v_cache + ((static_cast<long>(v_page[u]) * nkv + kh) * dv + f) * page_size + place_in_page(j, page_size, page_shift));
+                    v_cache + v_page[u] * v_page_stride + v_off[u] + place_in_page(j, page_size, page_shift));
                 if (j + E > kv) {         // places of the page that no token has written yet may hold anything
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
@@ -415,20 +443,18 @@ __global__ __launch_bounds__(64 * RT, (DT * RW <= 8 ? 2 : 1)) void window_attent
     };
     auto stash = [&]() {
 #pragma unroll
-        for (int u = 0; u < KU; ++u)
-            if (k_row[u] >= 0) *reinterpret_cast<w_u32x4*>(k_s + k_row[u] * krow + k_col[u] * E) = k_regs[u];
+        for (int u = 0; u < KU; ++u) {
+            if (u >= ku_n) break;
+            if (k_row[u] >= 0) *reinterpret_cast<w_u32x4*>(k_s + k_lds[u]) = k_regs[u];
+        }
 #pragma unroll
         for (int u = 0; u < VU; ++u) {
-            const int idx = tid + u * THREADS;
-            if (idx >= v_total) continue;
-            const int f = idx / VKP, v_key = (idx % VKP) * E;
+            if (v_key[u] < 0) continue;
             if constexpr (sizeof(T) == 4) {
-                *reinterpret_cast<w_u32x4*>(v_s + f * VROW + v_key) = v_regs[u];
+                *reinterpret_cast<w_u32x4*>(v_s + v_lds[u]) = v_regs[u];
             } else {
-                // in the order in which a lane takes them: within 32 keys (quarter of the wavefront, tile, key)
-                const int v_pos = (v_key / 32) * 32 + ((v_key % 16) / 4) * 8 + ((v_key % 32) / 16) * 4;
-                *reinterpret_cast<w_u32x2*>(v_s + f * VROW + v_pos) = w_u32x2{v_regs[u].x, v_regs[u].y};
-                *reinterpret_cast<w_u32x2*>(v_s + f * VROW + v_pos + 8) = w_u32x2{v_regs[u].z, v_regs[u].w};
+                *reinterpret_cast<w_u32x2*>(v_s + v_lds[u]) = w_u32x2{v_regs[u].x, v_regs[u].y};
+                *reinterpret_cast<w_u32x2*>(v_s + v_lds[u] + 8) = w_u32x2{v_regs[u].z, v_regs[u].w};
             }
         }
     };
@@ -470,25 +496,40 @@ __global__ __launch_bounds__(64 * RT, (DT * RW <= 8 ? 2 : 1)) void window_attent
 #pragma unroll
         for (int w = 0; w < RW; ++w) {
             float mx = -INFINITY;
+            // a chunk that every row of the tile sees whole (below the diagonal and inside the window, or all kept
+            // tokens) needs no mask
+            const bool whole = key0 + KT - 1 <= tile_p_min[w] && (key0 >= tile_lo_max[w] || key0 + KT <= a.keep_first);
+            if (whole) {
 #pragma unroll
-            for (int kt = 0; kt < NKT; ++kt)
+                for (int kt = 0; kt < NKT; ++kt)
 #pragma unroll
-                for (int v = 0; v < 4; ++v) {
-                    const int key = key0 + kt * 16 + lg * 4 + v;
-                    const bool seen = key <= p_row[w] && (key >= lo_row[w] || key < a.keep_first);
-                    const float sc = seen ? acc[w][kt][v] * scale : -INFINITY;
-                    acc[w][kt][v] = sc;
-                    mx = fmaxf(mx, sc);
-                }
+                    for (int v = 0; v < 4; ++v) {
+                        acc[w][kt][v] *= scale;
+                        mx = fmaxf(mx, acc[w][kt][v]);
+                    }
+            } else {
+#pragma unroll
+                for (int kt = 0; kt < NKT; ++kt)
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) {
+                        const int key = key0 + kt * 16 + lg * 4 + v;
+                        const bool seen = key <= p_row[w] && (key >= lo_row[w] || key < a.keep_first);
+                        const float sc = seen ? acc[w][kt][v] * scale : -INFINITY;
+                        acc[w][kt][v] = sc;
+                        mx = fmaxf(mx, sc);
+                    }
+            }
             mx = fmaxf(mx, __shfl_xor(mx, 16, kWave));
             mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
             const float m_new = fmaxf(m_run[w], mx);
             const float m_use = m_new == -INFINITY ? 0.f : m_new;      // a row that has seen nothing yet: every exp below is 0
-            const float alpha = __builtin_amdgcn_exp2f((m_run[w] - m_use) * kLog2e);
-            l_run[w] *= alpha;
+            if (__any(m_new != m_run[w])) {                             // (a factor of exactly 1 otherwise)
+                const float alpha = __builtin_amdgcn_exp2f((m_run[w] - m_use) * kLog2e);
+                l_run[w] *= alpha;
 #pragma unroll
-            for (int d = 0; d < DT; ++d) {
-                o[w][d][0] *= alpha; o[w][d][1] *= alpha; o[w][d][2] *= alpha; o[w][d][3] *= alpha;
+                for (int d = 0; d < DT; ++d) {
+                    o[w][d][0] *= alpha; o[w][d][1] *= alpha; o[w][d][2] *= alpha; o[w][d][3] *= alpha;
+                }
             }
             m_run[w] = m_new;
             float sum = 0.f;
