@@ -68,7 +68,7 @@ def test_every_cutting_agrees_with_plain(models, name, dtype):
     cuttings = {"whole": H.trace_whole(reqs), "last decoded": H.trace_last_decoded(reqs, 40), "portions": H.trace_portions(reqs),
                 "mixed": H.trace_mixed(reqs, seed=5, decode_tail=20)}
     for what, trace in cuttings.items():
-        for page_size in (16, 32) if what == "whole" else (16,):
+        for page_size in (16, 32, 48) if what == "whole" else (16, 48) if what == "mixed" else (16,):
             need = H.max_live_tokens(trace, 64)
             eng = engine(models[name], dtype, page_size=page_size, max_tokens=need, max_requests=4)
             rows = H.replay(eng, trace)

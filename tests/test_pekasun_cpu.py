@@ -166,3 +166,29 @@ def test_the_residual_stream_after_every_layer_run(models, emulated):
     eng = Engine.from_dir(models["A"], dtype="float32", device="cpu", page_size=4, max_tokens=64, max_requests=1)
     rows = H.replay(eng, H.trace_whole({"r0": tokens}))
     H.assert_rows_match(rows, {"r0": logits}, 1e-5, "streams")
+
+
+# ----------------------------------------------------------------------------- the attention kernel's shape rule
+def test_the_window_attention_rule_returns_what_the_kernel_takes():
+    """Over a grid of sizes: row tiles of 4 or 8, 1 to 64 splits, LDS within 160 KB; None exactly where a size is not
+    covered (then the general kernel runs)."""
+    from easy_gpt.cpp_amd.kernels.hip import HipKernels
+
+    rule = HipKernels._window_attention_shape
+    for elem in (2, 4):
+        for dk, dv in [(16, 32), (64, 64), (160, 128), (256, 192), (256, 256), (72, 16), (40, 24), (264, 64), (64, 272), (12, 16)]:
+            for t, b, max_q in [(1, 1, 1), (8, 8, 1), (64, 64, 1), (300, 3, 200), (2048, 1, 2048), (40000, 2, 32000)]:
+                for nq, nkv in [(14, 2), (16, 1), (3, 3)]:
+                    for window, keep in [(0, 0), (1024, 4), (7, 0)]:
+                        shape = rule(t, b, nq, nkv, dk, dv, 16, window, keep, max_q, 4096, elem)
+                        covered = dk % (16 // elem) == 0 and dk <= 256 and dv % 16 == 0 and dv <= 256
+                        assert (shape is not None) == covered, (elem, dk, dv)
+                        if shape is None:
+                            continue
+                        tiles, splits = shape
+                        assert tiles in (4, 8) and 1 <= splits <= 64
+                        chunk, e = (64, 8) if elem == 2 else (32, 4)
+                        krow = -(-dk // (4 * e)) * 4 * e + e
+                        dv_tiles = next(n for n in (2, 4, 6, 8, 12, 16) if n * 16 >= dv)
+                        assert ((16 * tiles + chunk) * krow + dv_tiles * 16 * (chunk + e)) * elem <= 160 * 1024
+            assert rule(8, 8, 4, 2, dk, dv, 40, 0, 0, 1, 512, elem) is None          # pages that are no multiple of 16
