@@ -81,7 +81,12 @@ CONFIG_E = {
         layer(attention(5, 5, 20, 12, 6, 0, -0.3), None),
     ],
 }
-CONFIGS = {"A": (CONFIG_A, 5), "B": (CONFIG_B, 6), "C": (CONFIG_C, 7), "E": (CONFIG_E, 9)}
+# latent layers without a rotated part (no positions enter at all), one on the other's weights
+CONFIG_F = {
+    "architecture": "Pekasun", "vocab": 99, "width": 48, "norm": {"eps": 1e-6},
+    "layers": [layer(latent(2, 8, 0, 8, 16, 5, 0.3), 32), layer(latent(2, 8, 0, 8, 16, 5, 0.3), 32, weights_of=0)],
+}
+CONFIGS = {"A": (CONFIG_A, 5), "B": (CONFIG_B, 6), "C": (CONFIG_C, 7), "E": (CONFIG_E, 9), "F": (CONFIG_F, 10)}
 
 
 def draw_weights(cfg: dict, seed: int, sharp: float = 3.0) -> dict[str, torch.Tensor]:

@@ -126,7 +126,7 @@ def test_pages_of_kept_first_tokens_are_never_given_back(page_size, window, keep
 
 
 # ----------------------------------------------------------------------------- the engine's bookkeeping
-@pytest.mark.parametrize("name", ["A", "B", "C", "E"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "E", "F"])
 def test_cuttings_agree_with_plain(models, emulated, name):
     cfg = PM.CONFIGS[name][0]
     reqs = H.make_requests(cfg["vocab"], [5, 41, 1, 23], seed=11)
