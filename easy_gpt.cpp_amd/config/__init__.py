@@ -1,4 +1,5 @@
 from .base import ConfigError, KeyReader, read_json
+from .nebanex import NebanexConfig
 from .pekasun import PekasunConfig
 from .qwen2 import Qwen2Config
 from .registry import (
@@ -15,6 +16,7 @@ __all__ = [
     "Architecture",
     "ConfigError",
     "KeyReader",
+    "NebanexConfig",
     "PekasunConfig",
     "Qwen2Config",
     "UnknownArchitectureError",

@@ -1,10 +1,11 @@
 // Softmax attention over the paged cache with separate key and value sizes, a window that keeps the first tokens,
-// and a sink in the softmax; ragged batches (prompt portions and single decoded tokens in one launch).
+// a sink in the softmax and a learned bias per head and distance; ragged batches (prompt portions and single decoded tokens in one launch).
 //
 // Query i of request b stands at position p = kv_len[b] - q_len[b] + i and sees key j if j <= p and
 // (window == 0 or p - j < window or j < keep_first).  score = (q . k) * scale over the key size dk; the softmax is
 // over the visible keys, and with a sink its denominator also holds exp(sink[head]), which has no key and no value
-// and is not scaled; the output is the weighted sum of the values of size dv.  Query head h reads key/value head
+// and is not scaled; with a distance bias [nq][far + 1] the score of key j gets bias[head][min(p - j, far)] added, unscaled;
+// the output is the weighted sum of the values of size dv.  Query head h reads key/value head
 // h / (nq / nkv).  Queries q [T][nq][dk]; keys in pages [page][kv head][offset][dk], values in pages
 // [page][kv head][dv][offset]; nothing that is not visible is read, so pages need no clearing and pages that a window
 // gave back are never touched.  Scores, softmax statistics and the output sum are float32.
@@ -70,7 +71,8 @@ __global__ __launch_bounds__(64 * kSimpleWaves) void window_attention_simple_ker
     const T* __restrict__ q, T* __restrict__ out, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
     const int32_t* __restrict__ block_table, int table_width, const int32_t* __restrict__ q_start,
     const int32_t* __restrict__ q_len, const int32_t* __restrict__ kv_len, int n_seqs, int nq, int nkv, int dk, int dv,
-    int page_size, float scale, int window, int keep_first, const float* __restrict__ sink) {
+    int page_size, float scale, int window, int keep_first, const float* __restrict__ sink,
+    const float* __restrict__ dist_bias, int dist_far) {
     constexpr int kMaxOwn = kWidest / kWave;
     __shared__ __attribute__((aligned(16))) float q_s[kWidest];
     __shared__ float part_ml[kSimpleWaves][2];
@@ -97,6 +99,7 @@ __global__ __launch_bounds__(64 * kSimpleWaves) void window_attention_simple_ker
             const long page = table[j / page_size];
             const T* kr = k_cache + ((page * nkv + kvh) * page_size + j % page_size) * dk;
             s = dot_row(q_s, kr, dk) * scale;
+            if (dist_bias) s += dist_bias[static_cast<size_t>(h) * (dist_far + 1) + min(p - j, dist_far)];
         }
         const float m_new = fmaxf(m_run, wave_max(s));       // finite: the chunk's first key is visible
         const float pj = vi < n_visible ? expf(s - m_new) : 0.f;
@@ -218,6 +221,8 @@ struct WindowArgs {
     const int32_t* q_len;
     const int32_t* kv_len;
     const float* sink;
+    const float* dist_bias;  // [nq][dist_far + 1] or null
+    int dist_far;
     int table_width, n_seqs, n_tokens, nq, nkv, dk, dv, page_size, window, keep_first, n_splits;
     int page_shift;          // log2 of the page size if that is a power of two, else -1
     float scale;
@@ -499,7 +504,25 @@ __global__ __launch_bounds__(64 * RT, (DT * RW <= 8 ? 2 : 1)) void window_attent
             // a chunk that every row of the tile sees whole (below the diagonal and inside the window, or all kept
             // tokens) needs no mask
             const bool whole = key0 + KT - 1 <= tile_p_min[w] && (key0 >= tile_lo_max[w] || key0 + KT <= a.keep_first);
-            if (whole) {
+            if (a.dist_bias != nullptr) {
+                // the bias of the row's head by distance; a chunk that lies `far` or more behind every row of the tile
+                // gets the table's last entry throughout
+                const float* brow = a.dist_bias + static_cast<size_t>(head[w]) * (a.dist_far + 1);
+                const bool all_far = whole && tile_p_min[w] - (key0 + KT - 1) >= a.dist_far;
+                const float b_far = brow[a.dist_far];
+#pragma unroll
+                for (int kt = 0; kt < NKT; ++kt)
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) {
+                        const int key = key0 + kt * 16 + lg * 4 + v;
+                        const bool seen = key <= p_row[w] && (key >= lo_row[w] || key < a.keep_first);
+                        float sc = -INFINITY;
+                        if (all_far) sc = fmaf(acc[w][kt][v], scale, b_far);
+                        else if (seen) sc = fmaf(acc[w][kt][v], scale, brow[min(p_row[w] - key, a.dist_far)]);
+                        acc[w][kt][v] = sc;
+                        mx = fmaxf(mx, sc);
+                    }
+            } else if (whole) {
 #pragma unroll
                 for (int kt = 0; kt < NKT; ++kt)
 #pragma unroll
@@ -685,10 +708,10 @@ extern "C" int egpt_window_attention(const void* q, void* out, const void* k_cac
                                      const int32_t* block_table, int table_width, const int32_t* q_start,
                                      const int32_t* q_len, const int32_t* kv_len, int n_seqs, int n_tokens, int nq,
                                      int nkv, int dk, int dv, int page_size, float scale, int window, int keep_first,
-                                     const float* sink, int dtype, void* stream) {
+                                     const float* sink, const float* dist_bias, int dist_far, int dtype, void* stream) {
     if (!q || !out || !k_cache || !v_cache || !block_table || !q_start || !q_len || !kv_len) return EGPT_BAD_ARGUMENT;
     if (n_seqs <= 0 || n_tokens < 0 || nq <= 0 || nkv <= 0 || nq % nkv != 0 || dk <= 0 || dv <= 0 || page_size <= 0 ||
-        table_width <= 0 || window < 0 || keep_first < 0 || (dtype != 0 && dtype != 1))
+        table_width <= 0 || window < 0 || keep_first < 0 || (dtype != 0 && dtype != 1) || (dist_bias && dist_far < 0))
         return EGPT_BAD_ARGUMENT;
     if (dk > kWidest || dv > kWidest || nq > 65535) return EGPT_UNSUPPORTED_SIZE;
     if (n_tokens == 0) return EGPT_OK;
@@ -698,12 +721,12 @@ extern "C" int egpt_window_attention(const void* q, void* out, const void* k_cac
         window_attention_simple_kernel<float><<<grid, kWave * kSimpleWaves, 0, s>>>(
             static_cast<const float*>(q), static_cast<float*>(out), static_cast<const float*>(k_cache),
             static_cast<const float*>(v_cache), block_table, table_width, q_start, q_len, kv_len, n_seqs, nq, nkv, dk,
-            dv, page_size, scale, window, keep_first, sink);
+            dv, page_size, scale, window, keep_first, sink, dist_bias, dist_far);
     else
         window_attention_simple_kernel<bf16_t><<<grid, kWave * kSimpleWaves, 0, s>>>(
             static_cast<const bf16_t*>(q), static_cast<bf16_t*>(out), static_cast<const bf16_t*>(k_cache),
             static_cast<const bf16_t*>(v_cache), block_table, table_width, q_start, q_len, kv_len, n_seqs, nq, nkv, dk,
-            dv, page_size, scale, window, keep_first, sink);
+            dv, page_size, scale, window, keep_first, sink, dist_bias, dist_far);
     EGPT_CHECK_LAUNCH();
     return EGPT_OK;
 }
@@ -712,12 +735,12 @@ extern "C" int egpt_window_attention_tiled(const void* q, void* out, float* part
                                            const void* v_cache, const int32_t* block_table, int table_width,
                                            const int32_t* q_start, const int32_t* q_len, const int32_t* kv_len, int n_seqs,
                                            int n_tokens, int nq, int nkv, int dk, int dv, int page_size, float scale,
-                                           int window, int keep_first, const float* sink, int n_splits, int row_tiles,
-                                           int dtype, void* stream) {
+                                           int window, int keep_first, const float* sink, const float* dist_bias,
+                                           int dist_far, int n_splits, int row_tiles, int dtype, void* stream) {
     if (!q || !out || !k_cache || !v_cache || !block_table || !q_start || !q_len || !kv_len) return EGPT_BAD_ARGUMENT;
     if (n_seqs <= 0 || n_tokens < 0 || nq <= 0 || nkv <= 0 || nq % nkv != 0 || dk <= 0 || dv <= 0 || page_size <= 0 ||
         table_width <= 0 || window < 0 || keep_first < 0 || n_splits < 1 || (dtype != 0 && dtype != 1) ||
-        (row_tiles != 4 && row_tiles != 8))
+        (row_tiles != 4 && row_tiles != 8) || (dist_bias && dist_far < 0))
         return EGPT_BAD_ARGUMENT;
     if (n_splits > 1 && (!part_o || !part_ml)) return EGPT_BAD_ARGUMENT;
     const int e = dtype == 0 ? 4 : 8;
@@ -727,6 +750,7 @@ extern "C" int egpt_window_attention_tiled(const void* q, void* out, float* part
     WindowArgs a;
     a.q = q; a.out = out; a.part_o = part_o; a.part_ml = part_ml; a.k_cache = k_cache; a.v_cache = v_cache;
     a.block_table = block_table; a.q_start = q_start; a.q_len = q_len; a.kv_len = kv_len; a.sink = sink;
+    a.dist_bias = dist_bias; a.dist_far = dist_far;
     a.table_width = table_width; a.n_seqs = n_seqs; a.n_tokens = n_tokens; a.nq = nq; a.nkv = nkv; a.dk = dk; a.dv = dv;
     a.page_size = page_size; a.window = window; a.keep_first = keep_first; a.n_splits = n_splits; a.scale = scale;
     a.page_shift = -1;

@@ -184,6 +184,77 @@ __global__ __launch_bounds__(256) void sigmoid_gate_kernel(const T* __restrict__
     out[idx] = from_float<T>(to_float(x[src]) * (1.0f / (1.0f + expf(-gate))));
 }
 
+
+// One workgroup per token of a product row [nq heads of dk | nkv heads of dk | nkv heads of dv | anything else]: the
+// bias [nq * dk + nkv * dk + nkv * dv] is added, the queries are RMS-normed over all heads at once (one statistic
+// over nq * dk values, a weight per value), and so are the keys (over nkv * dk); the queries are then multiplied by
+// 1 + coef * ln(floor((p + 1) / every) + 1) at position p (every == 0: no such factor).  Queries go to q_out
+// [T][nq * dk], keys and values to the pages at slots[t] (slots null: nothing is stored).
+template <typename T>
+__global__ __launch_bounds__(256) void whole_norm_store_kernel(
+    ProductView<T> proj, int row_width, const T* __restrict__ bias, T* __restrict__ q_out, const T* __restrict__ q_weight,
+    const T* __restrict__ k_weight, float eps, const int32_t* __restrict__ positions, float coef, int every,
+    const int32_t* __restrict__ slots, T* __restrict__ k_cache, T* __restrict__ v_cache, int nq, int nkv, int dk, int dv,
+    int page_size) {
+    __shared__ float scratch[16];
+    const int t = blockIdx.x;
+    const size_t row = static_cast<size_t>(t) * row_width;
+    const int qw = nq * dk, kw = nkv * dk, vw = nkv * dv;
+    float ssq = 0.f, ssk = 0.f;
+    for (int j = threadIdx.x; j < qw + kw; j += blockDim.x) {
+        float v = proj.at(row + j);
+        if (bias) v += to_float(bias[j]);
+        if (j < qw) ssq = fmaf(v, v, ssq); else ssk = fmaf(v, v, ssk);
+    }
+    float inv_q = 1.0f, inv_k = 1.0f;
+    if (q_weight) inv_q = inv_rms(block_sum(ssq, scratch), 1.0f / static_cast<float>(qw), eps);
+    if (k_weight) inv_k = inv_rms(block_sum(ssk, scratch), 1.0f / static_cast<float>(kw), eps);
+    if (every > 0) inv_q *= 1.0f + coef * logf(static_cast<float>((positions[t] + 1) / every + 1));
+    for (int j = threadIdx.x; j < qw; j += blockDim.x) {
+        float v = proj.at(row + j);
+        if (bias) v += to_float(bias[j]);
+        v *= inv_q;
+        if (q_weight) v *= to_float(q_weight[j]);
+        q_out[static_cast<size_t>(t) * qw + j] = from_float<T>(v);
+    }
+    if (slots == nullptr) return;
+    const long page = slots[t] / page_size;
+    const int off = slots[t] % page_size;
+    for (int j = threadIdx.x; j < kw; j += blockDim.x) {
+        float v = proj.at(row + qw + j);
+        if (bias) v += to_float(bias[qw + j]);
+        v *= inv_k;
+        if (k_weight) v *= to_float(k_weight[j]);
+        const int head = j / dk, d = j % dk;
+        k_cache[((page * nkv + head) * page_size + off) * dk + d] = from_float<T>(v);
+    }
+    for (int j = threadIdx.x; j < vw; j += blockDim.x) {
+        float v = proj.at(row + qw + kw + j);
+        if (bias) v += to_float(bias[qw + kw + j]);
+        const int head = j / dv, d = j % dv;
+        v_cache[((page * nkv + head) * dv + d) * page_size + off] = from_float<T>(v);
+    }
+}
+
+// out[t][h * dv + d] = x[t][h * dv + d] / rms(x[t][h * dv ..]) * weight[d] * silu(g[t][gate_off + h * dv + d]): the
+// RMS norm of every head's float32 output with a weight that the heads share, and a SiLU gate from columns of a
+// product row.  One wavefront per (token, head).
+template <typename T>
+__global__ __launch_bounds__(kWave) void head_norm_gate_kernel(const float* __restrict__ x, const T* __restrict__ weight,
+                                                               float eps, ProductView<T> g, int gate_width, int gate_off,
+                                                               T* __restrict__ out, int heads, int dv) {
+    const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+    const float* xr = x + (static_cast<size_t>(t) * heads + h) * dv;
+    float ss = 0.f;
+    for (int d = lane; d < dv; d += kWave) ss = fmaf(xr[d], xr[d], ss);
+    const float inv = inv_rms(wave_sum(ss), 1.0f / static_cast<float>(dv), eps);
+    for (int d = lane; d < dv; d += kWave) {
+        const float gate = g.at(static_cast<size_t>(t) * gate_width + gate_off + h * dv + d);
+        const float y = xr[d] * inv * to_float(weight[d]) * (gate / (1.0f + expf(-gate)));
+        out[(static_cast<size_t>(t) * heads + h) * dv + d] = from_float<T>(y);
+    }
+}
+
 template <typename T>
 static ProductView<T> view_of(const void* p, int n_splits, size_t split_stride) {
     ProductView<T> v;
@@ -303,6 +374,56 @@ extern "C" int egpt_sigmoid_gate(const void* x, int heads, const void* gate, int
         sigmoid_gate_kernel<bf16_t><<<blocks, 256, 0, s>>>(static_cast<const bf16_t*>(x), heads,
                                                            view_of<bf16_t>(gate, gate_splits, stride), factor, gate_width,
                                                            gate_off, static_cast<bf16_t*>(out), n_tokens, n);
+    EGPT_CHECK_LAUNCH();
+    return EGPT_OK;
+}
+
+extern "C" int egpt_whole_norm_store(const void* proj, int n_splits, int row_width, const void* bias, void* q_out,
+                                     const void* q_weight, const void* k_weight, float eps, const int32_t* positions,
+                                     float coef, int every, const int32_t* slots, void* k_cache, void* v_cache,
+                                     int n_tokens, int nq, int nkv, int dk, int dv, int page_size, int dtype, void* stream) {
+    if (!proj || !q_out || n_splits < 0 || n_tokens < 0 || nq <= 0 || nkv <= 0 || dk <= 0 || dv <= 0 || page_size <= 0 ||
+        every < 0 || (dtype != 0 && dtype != 1))
+        return EGPT_BAD_ARGUMENT;
+    if (row_width < (nq + nkv) * dk + nkv * dv) return EGPT_BAD_ARGUMENT;
+    if (every > 0 && !positions) return EGPT_BAD_ARGUMENT;
+    if (slots && (!k_cache || !v_cache)) return EGPT_BAD_ARGUMENT;
+    if (n_tokens == 0) return EGPT_OK;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const size_t stride = static_cast<size_t>(n_tokens) * row_width;
+    if (dtype == 0)
+        whole_norm_store_kernel<float><<<n_tokens, 256, 0, s>>>(
+            view_of<float>(proj, n_splits, stride), row_width, static_cast<const float*>(bias), static_cast<float*>(q_out),
+            static_cast<const float*>(q_weight), static_cast<const float*>(k_weight), eps, positions, coef, every, slots,
+            static_cast<float*>(k_cache), static_cast<float*>(v_cache), nq, nkv, dk, dv, page_size);
+    else
+        whole_norm_store_kernel<bf16_t><<<n_tokens, 256, 0, s>>>(
+            view_of<bf16_t>(proj, n_splits, stride), row_width, static_cast<const bf16_t*>(bias), static_cast<bf16_t*>(q_out),
+            static_cast<const bf16_t*>(q_weight), static_cast<const bf16_t*>(k_weight), eps, positions, coef, every, slots,
+            static_cast<bf16_t*>(k_cache), static_cast<bf16_t*>(v_cache), nq, nkv, dk, dv, page_size);
+    EGPT_CHECK_LAUNCH();
+    return EGPT_OK;
+}
+
+extern "C" int egpt_head_norm_gate(const float* x, const void* weight, float eps, const void* gate, int gate_splits,
+                                   int gate_width, int gate_off, void* out, int n_tokens, int heads, int dv, int dtype,
+                                   void* stream) {
+    if (!x || !weight || !gate || !out || n_tokens < 0 || heads <= 0 || dv <= 0 || gate_splits < 0 || gate_off < 0 ||
+        gate_off + heads * dv > gate_width || (dtype != 0 && dtype != 1))
+        return EGPT_BAD_ARGUMENT;
+    if (heads > 65535) return EGPT_UNSUPPORTED_SIZE;
+    if (n_tokens == 0) return EGPT_OK;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const size_t stride = static_cast<size_t>(n_tokens) * gate_width;
+    dim3 grid(n_tokens, heads);
+    if (dtype == 0)
+        head_norm_gate_kernel<float><<<grid, kWave, 0, s>>>(x, static_cast<const float*>(weight), eps,
+                                                            view_of<float>(gate, gate_splits, stride), gate_width, gate_off,
+                                                            static_cast<float*>(out), heads, dv);
+    else
+        head_norm_gate_kernel<bf16_t><<<grid, kWave, 0, s>>>(x, static_cast<const bf16_t*>(weight), eps,
+                                                             view_of<bf16_t>(gate, gate_splits, stride), gate_width, gate_off,
+                                                             static_cast<bf16_t*>(out), heads, dv);
     EGPT_CHECK_LAUNCH();
     return EGPT_OK;
 }

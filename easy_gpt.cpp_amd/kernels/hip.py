@@ -28,7 +28,7 @@ def _load_library() -> ctypes.CDLL:
         lib = ctypes.CDLL(path)
     except (build.BuildError, OSError) as e:
         raise KernelsUnavailable(f"the HIP kernel library could not be built or loaded: {e}") from e
-    if lib.egpt_abi_version() != 19:
+    if lib.egpt_abi_version() != 20:
         raise KernelsUnavailable(f"{path} has an unexpected ABI version")
     return lib
 
@@ -105,9 +105,22 @@ class HipKernels(KernelBackend):
             "egpt_head_norm_store": [vp, i, vp, i, i, f, vp, vp, vp, f, i, vp, vp, vp, i, i, i, i, i, i, i, vp],
             "egpt_latent_prep": [vp, i, vp, i, i, f, i, vp, vp, vp, f, vp, f, i, vp, vp, vp, i, i, i, i, i, i, i, vp],
             "egpt_sigmoid_gate": [vp, i, vp, i, vp, i, i, f, i, i, vp, i, i, i, vp],
-            "egpt_window_attention": [vp, vp, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, i, f, i, i, vp, i, vp],
-            "egpt_window_attention_tiled": [vp, vp, vp, vp, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, i, f, i, i, vp, i, i,
-                                            i, vp],
+            "egpt_window_attention": [vp, vp, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, i, f, i, i, vp, vp, i, i, vp],
+            "egpt_window_attention_tiled": [vp, vp, vp, vp, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, i, f, i, i, vp, vp, i,
+                                            i, i, i, vp],
+            "egpt_embed_scaled": [vp, vp, f, vp, i, i, i, i, vp],
+            "egpt_add_layernorm": [vp, vp, i, i, vp, vp, vp, f, vp, i, i, i, vp],
+            "egpt_normed_pair_mean": [vp, i, vp, i, vp, vp, vp, vp, f, f, vp, i, i, i, vp],
+            "egpt_tanh_cap": [vp, f, ctypes.c_longlong, vp],
+            "egpt_whole_norm_store": [vp, i, i, vp, vp, vp, vp, f, vp, f, i, vp, vp, vp, i, i, i, i, i, i, i, vp],
+            "egpt_head_norm_gate": [vp, vp, f, vp, i, i, i, vp, i, i, i, i, vp],
+            "egpt_channel_decay": [vp, i, i, i, i, vp, vp, f, vp, i, i, i, vp],
+            "egpt_decayed_state_scan": [vp, i, i, i, i, i, f, vp, vp, vp, vp, vp, vp, i, i, vp, i, i, i, i, vp],
+            "egpt_moe_route": [vp, vp, vp, vp, vp, i, i, i, i, i, vp],
+            "egpt_moe_group": [vp, vp, vp, vp, vp, i, i, i, i, vp],
+            "egpt_moe_gate_up": [vp, vp, vp, vp, vp, i, i, i, i, i, i, vp],
+            "egpt_moe_down": [vp, vp, vp, vp, i, i, i, i, i, i, vp],
+            "egpt_moe_combine": [vp, vp, vp, vp, i, i, i, vp],
         }
         lib.egpt_sample_workspace.restype = ctypes.c_size_t
         lib.egpt_sample_workspace.argtypes = [i, i]
@@ -943,7 +956,7 @@ class HipKernels(KernelBackend):
                   out.data_ptr(), t, n, dt, self._stream())
 
     def window_attention(self, q, out, k_cache, v_cache, block_table, q_start, q_len, kv_len, nq, nkv, dk, dv, page_size,
-                         scale, window, keep_first, sink, max_q_len, max_kv_len):
+                         scale, window, keep_first, sink, max_q_len, max_kv_len, dist_bias=None):
         t = q.shape[0]
         b, width = block_table.shape
         dt = self._act(q, "q")
@@ -955,6 +968,12 @@ class HipKernels(KernelBackend):
             self._need(v, name, _I32, (b,))
         if sink is not None:
             self._need(sink, "sink", _F32, (nq,))
+        dist_far = 0
+        if dist_bias is not None:
+            if dist_bias.dim() != 2 or dist_bias.shape[1] < 1:
+                raise ValueError("dist_bias must be [query heads, far + 1]")
+            self._need(dist_bias, "dist_bias", _F32, (nq, dist_bias.shape[1]))
+            dist_far = int(dist_bias.shape[1]) - 1
         if max_kv_len > width * page_size:
             raise ValueError(f"block table of width {width} cannot hold {max_kv_len} tokens at page size {page_size}")
         if dk > self.max_window_attention_dim or dv > self.max_window_attention_dim:
@@ -970,12 +989,194 @@ class HipKernels(KernelBackend):
             self._run("egpt_window_attention_tiled", q.data_ptr(), out.data_ptr(), self._ptr(part_o), self._ptr(part_ml),
                       k_cache.data_ptr(), v_cache.data_ptr(), block_table.data_ptr(), width, q_start.data_ptr(),
                       q_len.data_ptr(), kv_len.data_ptr(), b, t, nq, nkv, dk, dv, page_size, float(scale), int(window),
-                      int(keep_first), self._ptr(sink), n_splits, row_tiles, dt, self._stream())
+                      int(keep_first), self._ptr(sink), self._ptr(dist_bias), dist_far, n_splits, row_tiles, dt,
+                      self._stream())
             return
         # sizes that the matrix-core kernel does not take: the general kernel
         self._run("egpt_window_attention", q.data_ptr(), out.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
                   block_table.data_ptr(), width, q_start.data_ptr(), q_len.data_ptr(), kv_len.data_ptr(), b, t, nq, nkv,
-                  dk, dv, page_size, float(scale), int(window), int(keep_first), self._ptr(sink), dt, self._stream())
+                  dk, dv, page_size, float(scale), int(window), int(keep_first), self._ptr(sink), self._ptr(dist_bias),
+                  dist_far, dt, self._stream())
+
+
+    # ------------------------------------------------------------------ stream operations beyond the RMS norm
+    def embed_scaled(self, token_ids, table, factor, out):
+        dt = self._act(table, "table")
+        v, h = table.shape
+        t = token_ids.shape[0]
+        self._need(token_ids, "token_ids", _I32, (t,))
+        self._need(table, "table")
+        self._need(out, "out", _F32, (t, h))
+        self._run("egpt_embed_scaled", token_ids.data_ptr(), table.data_ptr(), float(factor), out.data_ptr(), t, h, v, dt,
+                  self._stream())
+
+    def add_layernorm(self, h, delta, rows, weight, bias, eps, out):
+        """h += delta (act [T, H] or float32 partial sums [S, T, H]; None: nothing), then the layer norm of every row
+        (rows None; h is written back) or of the rows listed in `rows` (h untouched) to `out`."""
+        dt = self._act(weight, "weight")
+        t, hidden = h.shape
+        self._need(h, "h", _F32)
+        self._need(weight, "weight", None, (hidden,))
+        if bias is not None:
+            self._need(bias, "bias", weight.dtype, (hidden,))
+        n = t if rows is None else rows.shape[0]
+        if rows is not None:
+            self._need(rows, "rows", _I32, (n,))
+        self._need(out, "out", weight.dtype, (n, hidden))
+        splits = 0 if delta is None else self._product(delta, "delta", weight.dtype, t, hidden)
+        self._run("egpt_add_layernorm", h.data_ptr(), self._ptr(delta), splits, t, self._ptr(rows), weight.data_ptr(),
+                  self._ptr(bias), float(eps), out.data_ptr(), n, hidden, dt, self._stream())
+
+    def normed_pair_mean(self, a, b, bias_a, bias_b, weight_a, weight_b, eps, factor):
+        """float32 [1, T, H]: factor * (rmsnorm(a + bias_a) * weight_a + rmsnorm(b + bias_b) * weight_b); a and b are
+        products (act [T, H] or float32 partial sums [S, T, H])."""
+        dt = self._act(weight_a, "weight_a")
+        t, hidden = a.shape[-2], a.shape[-1]
+        sa = self._product(a, "a", weight_a.dtype, t, hidden)
+        sb = self._product(b, "b", weight_a.dtype, t, hidden)
+        for name, w in (("weight_a", weight_a), ("weight_b", weight_b), ("bias_a", bias_a), ("bias_b", bias_b)):
+            if w is not None:
+                self._need(w, name, weight_a.dtype, (hidden,))
+        out = torch.empty((1, t, hidden), dtype=_F32, device=a.device)
+        self._run("egpt_normed_pair_mean", a.data_ptr(), sa, b.data_ptr(), sb, self._ptr(bias_a), self._ptr(bias_b),
+                  weight_a.data_ptr(), weight_b.data_ptr(), float(eps), float(factor), out.data_ptr(), t, hidden, dt,
+                  self._stream())
+        return out
+
+    def tanh_cap(self, x, cap):
+        self._need(x, "x", _F32)
+        self._run("egpt_tanh_cap", x.data_ptr(), float(cap), x.numel(), self._stream())
+
+    def whole_norm_store(self, proj, bias, q_out, q_weight, k_weight, eps, positions, coef, every, slots, k_cache, v_cache,
+                         nq, nkv, dk, dv, page_size):
+        t, width = proj.shape[-2], proj.shape[-1]
+        dt = self._act(q_out, "q_out")
+        used = (nq + nkv) * dk + nkv * dv
+        if width < used:
+            raise ValueError(f"proj rows of {width} values cannot hold {nq} + {nkv} heads of {dk} and {nkv} of {dv}")
+        splits = self._product(proj, "proj", q_out.dtype, t, width)
+        self._need(q_out, "q_out", None, (t, nq * dk))
+        if bias is not None:
+            self._need(bias, "bias", q_out.dtype, (used,))
+        if q_weight is not None:
+            self._need(q_weight, "q_weight", q_out.dtype, (nq * dk,))
+        if k_weight is not None:
+            self._need(k_weight, "k_weight", q_out.dtype, (nkv * dk,))
+        if every:
+            self._need(positions, "positions", _I32, (t,))
+        if slots is not None:
+            self._need(slots, "slots", _I32, (t,))
+            self._key_value_pages(k_cache, v_cache, q_out.dtype, nkv, page_size, dk, dv)
+        self._run("egpt_whole_norm_store", proj.data_ptr(), splits, int(width), self._ptr(bias), q_out.data_ptr(),
+                  self._ptr(q_weight), self._ptr(k_weight), float(eps), self._ptr(positions) if every else None, float(coef),
+                  int(every), self._ptr(slots), self._ptr(k_cache) if slots is not None else None,
+                  self._ptr(v_cache) if slots is not None else None, t, nq, nkv, dk, dv, page_size, dt, self._stream())
+
+    def head_norm_gate(self, x, weight, eps, gate, gate_offset, out, heads, dv):
+        t = out.shape[0]
+        dt = self._act(out, "out")
+        self._need(x, "x", _F32, (t, heads * dv))
+        self._need(out, "out", None, (t, heads * dv))
+        self._need(weight, "weight", out.dtype, (dv,))
+        width = gate.shape[-1]
+        splits = self._product(gate, "gate", out.dtype, t, width)
+        if gate_offset < 0 or gate_offset + heads * dv > width:
+            raise ValueError(f"gate columns {gate_offset}..{gate_offset + heads * dv} lie outside rows of {width} values")
+        self._run("egpt_head_norm_gate", x.data_ptr(), weight.data_ptr(), float(eps), gate.data_ptr(), splits, int(width),
+                  int(gate_offset), out.data_ptr(), t, heads, dv, dt, self._stream())
+
+    # ------------------------------------------------------------------ a decaying matrix state per head
+    def channel_decay(self, low, low_offset, rank, w, bias, tau):
+        t, width = low.shape[-2], low.shape[-1]
+        dt = self._act(w, "w")
+        channels = w.shape[0]
+        self._need(w, "w", None, (channels, rank))
+        if bias is not None:
+            self._need(bias, "bias", w.dtype, (channels,))
+        splits = self._product(low, "low", w.dtype, t, width)
+        if low_offset < 0 or low_offset + rank > width:
+            raise ValueError(f"columns {low_offset}..{low_offset + rank} lie outside rows of {width} values")
+        out = torch.empty((t, channels), dtype=_F32, device=w.device)
+        self._run("egpt_channel_decay", low.data_ptr(), splits, int(width), int(low_offset), int(rank), w.data_ptr(),
+                  self._ptr(bias), float(tau), out.data_ptr(), t, channels, dt, self._stream())
+        return out
+
+    def decayed_state_scan(self, proj, act_dtype, q_offset, k_offset, v_offset, q_scale, decay, states, slots, fresh, q_start,
+                           q_len, heads, dk, dv):
+        t, width = proj.shape[-2], proj.shape[-1]
+        if act_dtype not in _DT:
+            raise TypeError("act_dtype must be float32 or bfloat16")
+        splits = self._product(proj, "proj", act_dtype, t, width)
+        b = q_start.shape[0]
+        self._need(decay, "decay", _F32, (t, heads * dk))
+        self._need(states, "states", _F32)
+        if states.dim() != 4 or tuple(states.shape[1:]) != (heads, dk, dv):
+            raise ValueError(f"states must be [slots, {heads}, {dk}, {dv}], got {tuple(states.shape)}")
+        self._need(slots, "slots", _I32, (b,))
+        self._need(q_start, "q_start", _I32, (b,))
+        self._need(q_len, "q_len", _I32, (b,))
+        if fresh is not None:
+            self._need(fresh, "fresh", torch.bool, (b,))
+        for off, n in ((q_offset, heads * dk), (k_offset, heads * dk), (v_offset, heads * dv)):
+            if off < 0 or off + n > width:
+                raise ValueError(f"columns {off}..{off + n} lie outside rows of {width} values")
+        if dk > 256:
+            raise ValueError(f"key size {dk} is not supported by the state scan (at most 256)")
+        out = torch.empty((t, heads * dv), dtype=_F32, device=decay.device)
+        self._run("egpt_decayed_state_scan", proj.data_ptr(), splits, int(width), int(q_offset), int(k_offset), int(v_offset),
+                  float(q_scale), decay.data_ptr(), states.data_ptr(), slots.data_ptr(), self._ptr(fresh), q_start.data_ptr(),
+                  q_len.data_ptr(), b, t, out.data_ptr(), heads, dk, dv, _DT[act_dtype], self._stream())
+        return out
+
+    # ------------------------------------------------------------------ a mixture of experts
+    @staticmethod
+    def _moe_tile_rows(n_rows: int, experts: int) -> int:
+        """Rows to a tile of the grouped products: 16 while an expert gets few rows, 64 when it gets hundreds."""
+        per_expert = n_rows / max(experts, 1)
+        return 16 if per_expert <= 24 else (32 if per_expert <= 96 else 64)
+
+    def expert_mixture(self, x, router, router_bias, w_gate_up, w_down, top):
+        """float32 [T, H]: for every token the `top` experts with the largest float32 router logits (x router^T + bias),
+        weighted by the softmax over those logits; an expert is down(silu(gate x) * (up x)).  w_gate_up [E, 2 ff, H]
+        (an expert's gate rows, then its up rows), w_down [E, H, ff]."""
+        t, hidden = x.shape
+        dt = self._act(x, "x")
+        experts, ff2, _ = w_gate_up.shape
+        ff = ff2 // 2
+        self._need(x, "x")
+        self._need(router, "router", x.dtype, (experts, hidden))
+        if router_bias is not None:
+            self._need(router_bias, "router_bias", x.dtype, (experts,))
+        self._need(w_gate_up, "w_gate_up", x.dtype, (experts, 2 * ff, hidden))
+        self._need(w_down, "w_down", x.dtype, (experts, hidden, ff))
+        if not 0 < top <= experts:
+            raise ValueError(f"top ({top}) must be between 1 and the number of experts ({experts})")
+        if experts > 1024:
+            raise ValueError(f"{experts} experts are not supported (at most 1024)")
+        dev = x.device
+        n_rows = t * top
+        tile_rows = self._moe_tile_rows(n_rows, experts)
+        chosen = torch.empty((t, top), dtype=_I32, device=dev)
+        weight = torch.empty((t, top), dtype=_F32, device=dev)
+        row_token = torch.empty((n_rows,), dtype=_I32, device=dev)
+        place = torch.empty((t, top), dtype=_I32, device=dev)
+        tiles = torch.empty((1 + 3 * (n_rows // tile_rows + experts + 1),), dtype=_I32, device=dev)
+        counts = torch.empty((experts,), dtype=_I32, device=dev)
+        act = torch.empty((n_rows, ff), dtype=x.dtype, device=dev)
+        y = torch.empty((n_rows, hidden), dtype=_F32, device=dev)
+        out = torch.empty((t, hidden), dtype=_F32, device=dev)
+        st = self._stream()
+        self._run("egpt_moe_route", x.data_ptr(), router.data_ptr(), self._ptr(router_bias), chosen.data_ptr(),
+                  weight.data_ptr(), t, hidden, experts, top, dt, st)
+        self._run("egpt_moe_group", chosen.data_ptr(), row_token.data_ptr(), place.data_ptr(), tiles.data_ptr(),
+                  counts.data_ptr(), t, top, experts, tile_rows, st)
+        self._run("egpt_moe_gate_up", x.data_ptr(), w_gate_up.data_ptr(), row_token.data_ptr(), tiles.data_ptr(),
+                  act.data_ptr(), n_rows, hidden, ff, experts, tile_rows, dt, st)
+        self._run("egpt_moe_down", act.data_ptr(), w_down.data_ptr(), tiles.data_ptr(), y.data_ptr(), n_rows, hidden, ff,
+                  experts, tile_rows, dt, st)
+        self._run("egpt_moe_combine", y.data_ptr(), place.data_ptr(), weight.data_ptr(), out.data_ptr(), t, top, hidden, st)
+        self.last_routing = (chosen, weight)
+        return out
 
     wide_rows_from = 16384          # rows of a step from which the window attention gives a wavefront 32 of them,
     wide_rows_key_size = 192        # if its keys are wider than this

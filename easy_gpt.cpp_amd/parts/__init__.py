@@ -1,4 +1,4 @@
-from . import attention, block, embedding, feed_forward, head_attention, norm, position  # noqa: F401  (register the built-in parts)
+from . import attention, block, branch_mixers, embedding, expert_mixture, feed_forward, head_attention, norm, position  # noqa: F401  (register the built-in parts)
 from .base import (
     BLOCKS,
     FEED_FORWARDS,

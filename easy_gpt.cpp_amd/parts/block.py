@@ -27,6 +27,19 @@ class PreNormBlock(Block):
         return pending.h_after, m                                            # m is added by whoever comes next
 
 
+class PreNormMixerOnlyBlock(Block):
+    """The pre-norm arrangement of a layer that has no feed-forward: y = x + Mixer(N1(x))."""
+
+    norm_slots = ("mixer",)
+    uses_feed_forward = False
+
+    def forward(self, h, delta, ctx, cache, state):
+        pending = PendingNorm(h, delta, self.norms["mixer"])
+        x = pending if self.mixer.takes_pending_norm else pending.materialize()
+        a = self.mixer.forward(x, ctx, cache, state)
+        return pending.h_after, a
+
+
 class ParallelBlock(Block):
     """One norm whose output both branches read, both added to the stream: x = N(h); y = h + Mixer(x) + FF(x).
     The two branch outputs go on as one not-yet-added delta: float32 partial sums of both products side by side
@@ -87,5 +100,6 @@ class ParallelMixerOnlyBlock(ParallelBlock):
 
 
 register_part("block", "pre_norm", PreNormBlock)
+register_part("block", "pre_norm_mixer_only", PreNormMixerOnlyBlock)
 register_part("block", "parallel", ParallelBlock)
 register_part("block", "parallel_mixer_only", ParallelMixerOnlyBlock)

@@ -72,10 +72,28 @@ class NormedTokenEmbedding(TokenEmbedding):
         return out
 
 
+class ScaledTokenEmbedding(TokenEmbedding):
+    """x[t, :] = E[id_t, :] * scale, written as a float32 residual stream (the parts of a design that norms with a mean
+    read the stream in float32)."""
+
+    def __init__(self, prefix: str, hidden_size: int, vocab_size: int, scale: float, name: str = "weight"):
+        super().__init__(prefix, hidden_size, vocab_size, name)
+        self.scale = float(scale)
+
+    def forward(self, ctx) -> torch.Tensor:
+        token_ids = ctx.token_ids
+        out = torch.empty((token_ids.shape[0], self.hidden_size), device=token_ids.device, dtype=torch.float32)
+        kernels.backend().embed_scaled(token_ids, self.table, self.scale, out)
+        return out
+
+
 class LinearHead(OutputHead):
     graph_safe = True
 
-    def __init__(self, prefix: str, hidden_size: int, vocab_size: int, tied: bool, name: str = "weight"):
+    def __init__(self, prefix: str, hidden_size: int, vocab_size: int, tied: bool, name: str = "weight",
+                 softcap: float | None = None):
+        """softcap c: logits <- c * tanh(logits / c) (None: the product as it is)."""
+        self.softcap = float(softcap) if softcap else None
         self.prefix = prefix
         self.hidden_size = int(hidden_size)
         self.vocab_size = int(vocab_size)
@@ -101,9 +119,12 @@ class LinearHead(OutputHead):
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         out = torch.empty((x.shape[0], self.vocab_size), dtype=torch.float32, device=x.device)
         kernels.backend().linear(x, self.weight, None, out)
+        if self.softcap is not None:
+            kernels.backend().tanh_cap(out, self.softcap)
         return out
 
 
 register_part("embedding", "token_embedding", TokenEmbedding)
 register_part("embedding", "token_embedding_normed", NormedTokenEmbedding)
+register_part("embedding", "token_embedding_scaled", ScaledTokenEmbedding)
 register_part("output_head", "linear_head", LinearHead)

@@ -61,5 +61,44 @@ class ScalarRMSNorm(RMSNorm):
         self.weight = gain.expand(self.hidden_size).to(device).contiguous()
 
 
+class LayerNorm(Norm):
+    """y = (x - mean) / sqrt(var + eps) * weight + bias, var the mean of the squared deviations; statistics in float32,
+    fused with the addition into the residual stream like the RMS norm.  The weight is the tensor `prefix + name`, the
+    bias `prefix + bias_name` (None: the norm has no bias).  The stream it norms is float32."""
+
+    graph_safe = True
+
+    def __init__(self, prefix: str, hidden_size: int, eps: float, name: str = "weight", bias_name: str | None = "bias"):
+        self.prefix = prefix
+        self.hidden_size = int(hidden_size)
+        self.eps = float(eps)
+        self.name, self.bias_name = name, bias_name
+        self.weight: torch.Tensor | None = None
+        self.bias: torch.Tensor | None = None
+
+    def param_specs(self):
+        h = self.hidden_size
+        specs = [ParamSpec(self.prefix + self.name, (h,), role="norm_scale")]
+        if self.bias_name is not None:
+            specs.append(ParamSpec(self.prefix + self.bias_name, (h,), role="bias"))
+        return specs
+
+    def load(self, get, dtype, device):
+        self.weight = self._to(get(self.prefix + self.name), "compute", dtype, device)
+        if self.bias_name is not None:
+            self.bias = self._to(get(self.prefix + self.bias_name), "compute", dtype, device)
+
+    def forward(self, h, delta):
+        out = torch.empty(h.shape, dtype=self.weight.dtype, device=h.device)
+        kernels.backend().add_layernorm(h, delta, None, self.weight, self.bias, self.eps, out)
+        return out
+
+    def forward_rows(self, h, delta, rows):
+        out = torch.empty((rows.shape[0], h.shape[1]), dtype=self.weight.dtype, device=h.device)
+        kernels.backend().add_layernorm(h, delta, rows, self.weight, self.bias, self.eps, out)
+        return out
+
+
 register_part("norm", "rmsnorm", RMSNorm)
+register_part("norm", "layernorm", LayerNorm)
 register_part("norm", "rmsnorm_scalar", ScalarRMSNorm)

@@ -20,6 +20,9 @@ class ParamSpec:
     dtype   'compute' (cast to the engine's dtype), 'float32' or 'int32' (kept as stored)
     alt_shapes  other shapes accepted on load (the reference accepts [H, 1] for a
             norm weight, /root/reference/src/models/model_param_validation.cpp:62-74)
+    free_axes   axes whose length the stored tensor decides (a table's number of rows, a low-rank projection's
+            rank, where the configuration does not name them): any length of one or more is accepted there, and
+            `shape` gives the length that random weights draw
     """
 
     name: str
@@ -27,6 +30,7 @@ class ParamSpec:
     role: str = "matrix"
     dtype: str = "compute"
     alt_shapes: tuple[tuple[int, ...], ...] = ()
+    free_axes: tuple[int, ...] = ()
 
 
 @dataclass(frozen=True)

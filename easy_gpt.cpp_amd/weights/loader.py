@@ -34,6 +34,13 @@ class WeightsError(RuntimeError):
         self.wrong_shape = list(wrong_shape)
 
 
+def _fits_free_axes(shape: tuple[int, ...], spec: ParamSpec) -> bool:
+    """Whether `shape` is the declared one on every axis but those whose length the stored tensor decides."""
+    if not spec.free_axes or len(shape) != len(spec.shape):
+        return False
+    return all((a in spec.free_axes and n >= 1) or n == m for a, (n, m) in enumerate(zip(shape, spec.shape)))
+
+
 def check_names_and_shapes(
     available: dict[str, tuple[int, ...]],
     specs: Iterable[ParamSpec],
@@ -55,7 +62,7 @@ def check_names_and_shapes(
     for name, spec in declared.items():
         if name in available:
             shape = tuple(available[name])
-            if shape != tuple(spec.shape) and shape not in spec.alt_shapes:
+            if shape != tuple(spec.shape) and shape not in spec.alt_shapes and not _fits_free_axes(shape, spec):
                 wrong.append((name, shape, tuple(spec.shape)))
     if missing or unexpected or wrong:
         lines = [f"{where} does not match the model:"]
