@@ -177,7 +177,7 @@ class EmulatedKernels(KernelBackend):
         out.copy_((xx * torch.sigmoid(g)).to(out.dtype))
 
     def window_attention(self, q, out, k_cache, v_cache, block_table, q_start, q_len, kv_len, nq, nkv, dk, dv, page_size,
-                         scale, window, keep_first, sink, max_q_len, max_kv_len):
+                         scale, window, keep_first, sink, max_q_len, max_kv_len, dist_bias=None):
         group = nq // nkv
         q_all = q.view(q.shape[0], nq, dk).to(F64)
         for b in range(q_start.shape[0]):
@@ -194,10 +194,109 @@ class EmulatedKernels(KernelBackend):
                     keys = k_cache[pages, kh, offs, :].to(F64)
                     vals = v_cache[pages, kh, :, offs].to(F64)
                     sc = (keys @ q_all[s + i, h]) * scale
+                    if dist_bias is not None:
+                        sc = sc + dist_bias[h, (p - js).clamp(max=dist_bias.shape[1] - 1)].to(F64)
                     m = sc.max() if sink is None else torch.maximum(sc.max(), sink[h].to(F64))
                     e = torch.exp(sc - m)
                     denom = e.sum() + (torch.exp(sink[h].to(F64) - m) if sink is not None else 0.0)
                     out[s + i, h * dv : (h + 1) * dv] = ((e / denom) @ vals).to(out.dtype)
+
+    # ---- operations of designs with layer norms, side-by-side mixers, a decaying state and experts
+    def embed_scaled(self, token_ids, table, factor, out):
+        out.copy_((table[token_ids.long()].to(F64) * factor).to(out.dtype))
+
+    def add_layernorm(self, h, delta, rows, weight, bias, eps, out):
+        delta = _whole(delta)
+        if rows is None:
+            if delta is not None:
+                h.add_(delta.to(h.dtype))
+            x = h.to(F64)
+        else:
+            x = h[rows.long()].to(F64)
+            if delta is not None:
+                x = (h[rows.long()] + delta[rows.long()].to(h.dtype)).to(F64)
+        mu = x.mean(-1, keepdim=True)
+        y = (x - mu) / torch.sqrt(((x - mu) ** 2).mean(-1, keepdim=True) + eps) * weight.to(F64)
+        out.copy_((y if bias is None else y + bias.to(F64)).to(out.dtype))
+
+    def normed_pair_mean(self, a, b, bias_a, bias_b, weight_a, weight_b, eps, factor):
+        def normed(x, bias, w):
+            x = _whole(x).to(F64)
+            if bias is not None:
+                x = x + bias.to(F64)
+            return x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps) * w.to(F64)
+
+        return (factor * (normed(a, bias_a, weight_a) + normed(b, bias_b, weight_b))).to(torch.float32)[None]
+
+    def tanh_cap(self, x, cap):
+        x.copy_((cap * torch.tanh(x.to(F64) / cap)).to(x.dtype))
+
+    def whole_norm_store(self, proj, bias, q_out, q_weight, k_weight, eps, positions, coef, every, slots, k_cache, v_cache,
+                         nq, nkv, dk, dv, page_size):
+        x = _whole(proj).to(F64)
+        t = x.shape[0]
+        used = (nq + nkv) * dk + nkv * dv
+        x = x[:, :used] + (bias.to(F64) if bias is not None else 0.0)
+        unit = lambda a: a / torch.sqrt((a * a).mean(-1, keepdim=True) + eps)
+        q, k, v = x[:, : nq * dk], x[:, nq * dk : (nq + nkv) * dk], x[:, (nq + nkv) * dk :]
+        if q_weight is not None:
+            q = unit(q) * q_weight.to(F64)
+        if k_weight is not None:
+            k = unit(k) * k_weight.to(F64)
+        if every:
+            q = q * (1.0 + coef * torch.log(((positions.long() + 1) // every + 1).to(F64)))[:, None]
+        q_out.copy_(q.to(q_out.dtype))
+        if slots is not None:
+            self._store(k_cache, v_cache, slots, page_size, k.reshape(t, nkv, dk), v.reshape(t, nkv, dv))
+
+    def head_norm_gate(self, x, weight, eps, gate, gate_offset, out, heads, dv):
+        t = out.shape[0]
+        xx = x.to(F64).view(t, heads, dv)
+        xx = xx / torch.sqrt((xx * xx).mean(-1, keepdim=True) + eps) * weight.to(F64)
+        g = _whole(gate)[:, gate_offset : gate_offset + heads * dv].to(F64)
+        out.copy_((xx.reshape(t, heads * dv) * g * torch.sigmoid(g)).to(out.dtype))
+
+    def channel_decay(self, low, low_offset, rank, w, bias, tau):
+        z = _whole(low)[:, low_offset : low_offset + rank].to(F64) @ w.to(F64).T
+        if bias is not None:
+            z = z + bias.to(F64)
+        return (torch.sigmoid(z) ** (1.0 / tau)).to(torch.float32)
+
+    def decayed_state_scan(self, proj, act_dtype, q_offset, k_offset, v_offset, q_scale, decay, states, slots, fresh, q_start,
+                           q_len, heads, dk, dv):
+        x = _whole(proj).to(F64)
+        t = x.shape[0]
+        out = torch.zeros((t, heads * dv), dtype=torch.float32)
+        for b in range(q_start.shape[0]):
+            s0, n, slot = int(q_start[b]), int(q_len[b]), int(slots[b])
+            if n <= 0:
+                continue
+            st = torch.zeros((heads, dk, dv), dtype=F64) if fresh is not None and bool(fresh[b]) else states[slot].to(F64)
+            for i in range(s0, s0 + n):
+                q = x[i, q_offset : q_offset + heads * dk].view(heads, dk) * q_scale
+                k = x[i, k_offset : k_offset + heads * dk].view(heads, dk)
+                v = x[i, v_offset : v_offset + heads * dv].view(heads, dv)
+                st = decay[i].to(F64).view(heads, dk)[:, :, None] * st + k[:, :, None] * v[:, None, :]
+                out[i] = torch.einsum("hkv,hk->hv", st, q).reshape(-1).to(torch.float32)
+            states[slot] = st.to(states.dtype)
+        return out
+
+    def expert_mixture(self, x, router, router_bias, w_gate_up, w_down, top):
+        xx = x.to(F64)
+        z = xx @ router.to(F64).T
+        if router_bias is not None:
+            z = z + router_bias.to(F64)
+        val, idx = torch.topk(z, top, dim=-1)
+        wt = torch.softmax(val, dim=-1)
+        ff = w_gate_up.shape[1] // 2
+        out = torch.zeros(x.shape, dtype=F64)
+        for t in range(x.shape[0]):
+            for c in range(top):
+                e = int(idx[t, c])
+                gu = w_gate_up[e].to(F64) @ xx[t]
+                act = (gu[:ff] * torch.sigmoid(gu[:ff]) * gu[ff:]).to(x.dtype).to(F64)
+                out[t] += wt[t, c] * (w_down[e].to(F64) @ act)
+        return out.to(torch.float32)
 
     def swiglu(self, gate_up, out):
         gate_up = _whole(gate_up)

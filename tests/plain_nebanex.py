@@ -99,7 +99,8 @@ def biased_attention(h, w, p, m, eps):
     v = h @ w[p + "v"].T + w[p + "v.b"]
     q = rms_norm(q, w[p + "q.norm"], eps)                    # over the whole projection, all heads at once
     k = rms_norm(k, w[p + "k.norm"], eps)
-    q = q * query_factor(range(t), m["q_temp"]["coef"], m["q_temp"]["every"])[:, None]
+    if m.get("q_temp") is not None:
+        q = q * query_factor(range(t), m["q_temp"]["coef"], m["q_temp"]["every"])[:, None]
     q, k, v = q.view(t, nq, dk), k.view(t, nkv, dk), v.view(t, nkv, dv)
     bias = distance_bias(t, w[p + "rel"], m["bias_max"])
     causal = torch.ones(t, t).tril().bool()
