@@ -397,6 +397,42 @@ def pekasun_config(width, inner, heads, kv_heads, hd, rank, rot, window) -> dict
             "layers": [latent, plain] * (DESIGN_LAYERS // 2)}
 
 
+# `--design nebanex`: the Nebanex design (attention with a distance bias beside linear attention with a decaying
+# state, a mixture of experts with a shared expert) beside the Qwen2 model of the same width, depth, heads and head
+# size whose inner width is what a Nebanex token uses (its chosen experts and the shared one).  (label, width, heads,
+# kv heads, head size, state heads, state key size, state value size, experts, chosen, an expert's inner width,
+# the shared expert's)
+NEBANEX_SIZES = (
+    ("w896", 896, 14, 2, 64, 7, 64, 128, 16, 4, 1024, 768),
+    ("w2048", 2048, 16, 4, 128, 16, 64, 128, 32, 4, 1536, 2048),
+)
+
+
+def nebanex_config(width, heads, kv_heads, hd, s_heads, s_dim, s_vdim, experts, top, ff, shared) -> dict:
+    layer = {"type": "parallel",
+             "mixer": {"left": {"heads": heads, "kv_heads": kv_heads, "dim": hd, "vdim": hd, "scale": hd ** -0.5, "bias_max": 512,
+                                "q_temp": {"coef": 0.1, "every": 1024}},
+                       "right": {"heads": s_heads, "dim": s_dim, "vdim": s_vdim, "tau": 16.0}},
+             "mlp": {"kind": "moe", "router": {"experts": experts, "top": top}, "expert": {"ff": ff}, "shared": {"ff": shared}}}
+    return {"architecture": "Nebanex", "vocab": DESIGN_VOCAB, "width": width, "norm": {"eps": 1e-6}, "embedding": {"scale": 1.0},
+            "logit_softcap": 30.0, "layers": [layer] * DESIGN_LAYERS}
+
+
+def design_models(design):
+    """(label, {name: config}) for every size of the comparison, and how the sizes are named in the record."""
+    if design == "pekasun":
+        keys = ("width", "inner", "heads", "kv_heads", "head", "latent", "rotated", "window")
+        for s in DESIGN_SIZES:
+            label, width, inner, heads, kv_heads, hd = s[:6]
+            yield label, dict(zip(keys, s[1:])), pekasun_config(*s[1:]), (width, inner, heads, kv_heads, hd)
+    else:
+        keys = ("width", "heads", "kv_heads", "head", "state_heads", "state_key", "state_value", "experts", "chosen",
+                "expert_inner", "shared_inner")
+        for s in NEBANEX_SIZES:
+            label, width, heads, kv_heads, hd = s[:5]
+            yield label, dict(zip(keys, s[1:])), nebanex_config(*s[1:]), (width, s[9] * s[10] + s[11], heads, kv_heads, hd)
+
+
 def design_comparison(args) -> dict:
     import torch
 
@@ -406,9 +442,11 @@ def design_comparison(args) -> dict:
 
     g = torch.Generator().manual_seed(0)
     prefix, points = 2048, {}
-    for label, width, inner, heads, kv_heads, hd, rank, rot, window in DESIGN_SIZES:
+    design, sizes = args.design, {}
+    for label, named, design_cfg, (width, inner, heads, kv_heads, hd) in design_models(design):
+        sizes[label] = named
         models = {
-            "pekasun": pekasun_config(width, inner, heads, kv_heads, hd, rank, rot, window),
+            design: design_cfg,
             "qwen2": dict(QWEN25_05B, hidden_size=width, intermediate_size=inner, num_attention_heads=heads,
                           num_key_value_heads=kv_heads, head_dim=hd, num_hidden_layers=DESIGN_LAYERS, vocab_size=DESIGN_VOCAB,
                           tie_word_embeddings=False),
@@ -434,13 +472,12 @@ def design_comparison(args) -> dict:
             torch.cuda.empty_cache()
     first = DESIGN_SIZES[0][0]
     return {
-        "metric": "decode tokens/s of the Pekasun design at batch 8 behind 2,048 tokens (4 layers of width 896)",
-        "value": points[f"{first}_pekasun_decode_b8_tokens_per_s"], "unit": "tokens/s", "n_gpus": 1,
+        "metric": f"decode tokens/s of the {design.capitalize()} design at batch 8 behind 2,048 tokens (4 layers of width 896)",
+        "value": points[f"{first}_{design}_decode_b8_tokens_per_s"], "unit": "tokens/s", "n_gpus": 1,
         "higher_is_better": True, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
         "data": "synthetic: uniform-random token ids, random weights N(0, 0.02) from seed 0",
         "config": {"layers": DESIGN_LAYERS, "vocab": DESIGN_VOCAB, "prefix": prefix, "prefill_tokens": PREFILL_TOKENS,
-                   "sizes": {s[0]: dict(zip(("width", "inner", "heads", "kv_heads", "head", "latent", "rotated", "window"), s[1:]))
-                             for s in DESIGN_SIZES}},
+                   "sizes": sizes},
         "points": points,
     }
 
@@ -475,7 +512,7 @@ def main() -> int:
     ap.add_argument("--no-lookahead", action="store_true",
                     help="wait for a step's tokens on the host before the next step is launched (the scheduler with --serve, "
                          "the decode loop otherwise)")
-    ap.add_argument("--design", default=None, choices=["pekasun"],
+    ap.add_argument("--design", default=None, choices=["pekasun", "nebanex"],
                     help="instead of the record: prefill and decode of that design at a few layer sizes beside the Qwen2 "
                          "model of equal sizes")
     ap.add_argument("--direct-loop", action="store_true",

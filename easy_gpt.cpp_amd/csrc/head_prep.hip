@@ -200,39 +200,73 @@ __global__ __launch_bounds__(256) void whole_norm_store_kernel(
     const int t = blockIdx.x;
     const size_t row = static_cast<size_t>(t) * row_width;
     const int qw = nq * dk, kw = nkv * dk, vw = nkv * dv;
+    // a row of up to kKeep values per thread stays in registers between the statistics and the stores (all of a thread's
+    // loads in flight together); wider rows are read twice
+    constexpr int kKeep = 16;
+    const bool kept = qw + kw + vw <= kKeep * static_cast<int>(blockDim.x);
+    float val[kKeep];
     float ssq = 0.f, ssk = 0.f;
-    for (int j = threadIdx.x; j < qw + kw; j += blockDim.x) {
-        float v = proj.at(row + j);
-        if (bias) v += to_float(bias[j]);
-        if (j < qw) ssq = fmaf(v, v, ssq); else ssk = fmaf(v, v, ssk);
+    if (kept) {
+#pragma unroll
+        for (int i = 0; i < kKeep; ++i) {
+            const int j = threadIdx.x + i * blockDim.x;
+            val[i] = 0.f;
+            if (j < qw + kw + vw) {
+                val[i] = proj.at(row + j);
+                if (bias) val[i] += to_float(bias[j]);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < kKeep; ++i) {
+            const int j = threadIdx.x + i * blockDim.x;
+            if (j < qw) ssq = fmaf(val[i], val[i], ssq); else if (j < qw + kw) ssk = fmaf(val[i], val[i], ssk);
+        }
+    } else {
+        for (int j = threadIdx.x; j < qw + kw; j += blockDim.x) {
+            float v = proj.at(row + j);
+            if (bias) v += to_float(bias[j]);
+            if (j < qw) ssq = fmaf(v, v, ssq); else ssk = fmaf(v, v, ssk);
+        }
     }
     float inv_q = 1.0f, inv_k = 1.0f;
     if (q_weight) inv_q = inv_rms(block_sum(ssq, scratch), 1.0f / static_cast<float>(qw), eps);
     if (k_weight) inv_k = inv_rms(block_sum(ssk, scratch), 1.0f / static_cast<float>(kw), eps);
     if (every > 0) inv_q *= 1.0f + coef * logf(static_cast<float>((positions[t] + 1) / every + 1));
-    for (int j = threadIdx.x; j < qw; j += blockDim.x) {
-        float v = proj.at(row + j);
-        if (bias) v += to_float(bias[j]);
-        v *= inv_q;
-        if (q_weight) v *= to_float(q_weight[j]);
-        q_out[static_cast<size_t>(t) * qw + j] = from_float<T>(v);
+    long page = 0;
+    int off = 0;
+    if (slots != nullptr) {
+        page = slots[t] / page_size;
+        off = slots[t] % page_size;
     }
-    if (slots == nullptr) return;
-    const long page = slots[t] / page_size;
-    const int off = slots[t] % page_size;
-    for (int j = threadIdx.x; j < kw; j += blockDim.x) {
-        float v = proj.at(row + qw + j);
-        if (bias) v += to_float(bias[qw + j]);
-        v *= inv_k;
-        if (k_weight) v *= to_float(k_weight[j]);
-        const int head = j / dk, d = j % dk;
-        k_cache[((page * nkv + head) * page_size + off) * dk + d] = from_float<T>(v);
-    }
-    for (int j = threadIdx.x; j < vw; j += blockDim.x) {
-        float v = proj.at(row + qw + kw + j);
-        if (bias) v += to_float(bias[qw + kw + j]);
-        const int head = j / dv, d = j % dv;
-        v_cache[((page * nkv + head) * dv + d) * page_size + off] = from_float<T>(v);
+    auto put = [&](int j, float v) {
+        if (j < qw) {
+            v *= inv_q;
+            if (q_weight) v *= to_float(q_weight[j]);
+            q_out[static_cast<size_t>(t) * qw + j] = from_float<T>(v);
+        } else if (slots == nullptr) {
+            return;
+        } else if (j < qw + kw) {
+            const int jj = j - qw;
+            v *= inv_k;
+            if (k_weight) v *= to_float(k_weight[jj]);
+            k_cache[((page * nkv + jj / dk) * page_size + off) * dk + jj % dk] = from_float<T>(v);
+        } else {
+            const int jj = j - qw - kw;
+            v_cache[((page * nkv + jj / dv) * dv + jj % dv) * page_size + off] = from_float<T>(v);
+        }
+    };
+    if (kept) {
+#pragma unroll
+        for (int i = 0; i < kKeep; ++i) {
+            const int j = threadIdx.x + i * blockDim.x;
+            if (j < qw + kw + vw) put(j, val[i]);
+        }
+    } else {
+        for (int j = threadIdx.x; j < qw + kw + vw; j += blockDim.x) {
+            float v = proj.at(row + j);
+            if (bias) v += to_float(bias[j]);
+            put(j, v);
+        }
     }
 }
 

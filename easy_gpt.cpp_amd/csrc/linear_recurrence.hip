@@ -44,7 +44,7 @@ __global__ __launch_bounds__(256) void channel_decay_kernel(ProductView<T> low, 
     }
 }
 
-constexpr int kScanTokens = 8;      // tokens staged in LDS at a time
+constexpr int kScanTokens = 16;     // tokens staged in LDS at a time
 constexpr int kScanCols = 64;       // value channels per workgroup
 
 // One workgroup of four wavefronts per (request, head, 64 value channels).  A wavefront takes 16 value channels; its
@@ -80,49 +80,70 @@ __global__ __launch_bounds__(256) void decayed_state_scan_kernel(
         s[i] = (!start_anew && has_col && r < dk) ? state[static_cast<size_t>(r) * dv + j] : 0.f;
     }
     const int channels = heads * dk;
+    // The next tokens' queries, keys, decays and values travel through registers: their loads are issued before this
+    // batch of tokens is computed and stored to LDS behind it, so that a batch waits for memory once, not once per
+    // array, and not at all while the recurrence runs long.
+    constexpr int QKA = kScanTokens * 4 * DKR / 256, VL = kScanTokens * kScanCols / 256;
+    float rq[QKA], rk[QKA], ra[QKA], rv[VL];
+    auto fetch = [&](int base) {
+        const int count = min(kScanTokens, n - base);
+#pragma unroll
+        for (int u = 0; u < QKA; ++u) {
+            const int idx = tid + u * 256;
+            const int tt = idx / (4 * DKR), r = idx % (4 * DKR);
+            rq[u] = rk[u] = ra[u] = 0.f;
+            if (tt < count && r < dk) {
+                const size_t row = static_cast<size_t>(t0 + base + tt);
+                rq[u] = proj.at(row * proj_width + q_off + h * dk + r) * q_scale;
+                rk[u] = proj.at(row * proj_width + k_off + h * dk + r);
+                ra[u] = decay[row * channels + h * dk + r];
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < VL; ++u) {
+            const int idx = tid + u * 256;
+            const int tt = idx / kScanCols, c = idx % kScanCols;
+            rv[u] = 0.f;
+            if (tt < count && col0 + c < dv)
+                rv[u] = proj.at(static_cast<size_t>(t0 + base + tt) * proj_width + v_off + h * dv + col0 + c);
+        }
+    };
+    fetch(0);
     for (int base = 0; base < n; base += kScanTokens) {
         const int count = min(kScanTokens, n - base);
         __syncthreads();                          // the tokens before are read
-        for (int idx = tid; idx < kScanTokens * 4 * DKR; idx += 256) {
+#pragma unroll
+        for (int u = 0; u < QKA; ++u) {
+            const int idx = tid + u * 256;
             const int tt = idx / (4 * DKR), r = idx % (4 * DKR);
             const int at = tt * TOK + (r / DKR) * ROW + r % DKR;
-            float qv = 0.f, kv = 0.f, av = 0.f;
-            if (tt < count && r < dk) {
-                const size_t row = static_cast<size_t>(t0 + base + tt);
-                qv = proj.at(row * proj_width + q_off + h * dk + r) * q_scale;
-                kv = proj.at(row * proj_width + k_off + h * dk + r);
-                av = decay[row * channels + h * dk + r];
-            }
-            q_s[at] = qv;
-            k_s[at] = kv;
-            a_s[at] = av;
+            q_s[at] = rq[u];
+            k_s[at] = rk[u];
+            a_s[at] = ra[u];
         }
-        for (int idx = tid; idx < kScanTokens * kScanCols; idx += 256) {
-            const int tt = idx / kScanCols, c = idx % kScanCols;
-            float vv = 0.f;
-            if (tt < count && col0 + c < dv)
-                vv = proj.at(static_cast<size_t>(t0 + base + tt) * proj_width + v_off + h * dv + col0 + c);
-            v_s[idx] = vv;
-        }
+#pragma unroll
+        for (int u = 0; u < VL; ++u) v_s[tid + u * 256] = rv[u];
         __syncthreads();
+        if (base + kScanTokens < n) fetch(base + kScanTokens);
         for (int tt = 0; tt < count; ++tt) {
             const float vj = v_s[tt * kScanCols + col];
             const float4* a4 = reinterpret_cast<const float4*>(a_s + tt * TOK + slice * ROW);
             const float4* k4 = reinterpret_cast<const float4*>(k_s + tt * TOK + slice * ROW);
             const float4* q4 = reinterpret_cast<const float4*>(q_s + tt * TOK + slice * ROW);
-            float o = 0.f;
+            float o0 = 0.f, o1 = 0.f, o2 = 0.f, o3 = 0.f;       // four sums, so that no addition waits for the one before
 #pragma unroll
             for (int i = 0; i < DKR / 4; ++i) {
                 const float4 a = a4[i], k = k4[i], q = q4[i];
                 s[4 * i] = fmaf(a.x, s[4 * i], k.x * vj);
-                o = fmaf(s[4 * i], q.x, o);
+                o0 = fmaf(s[4 * i], q.x, o0);
                 s[4 * i + 1] = fmaf(a.y, s[4 * i + 1], k.y * vj);
-                o = fmaf(s[4 * i + 1], q.y, o);
+                o1 = fmaf(s[4 * i + 1], q.y, o1);
                 s[4 * i + 2] = fmaf(a.z, s[4 * i + 2], k.z * vj);
-                o = fmaf(s[4 * i + 2], q.z, o);
+                o2 = fmaf(s[4 * i + 2], q.z, o2);
                 s[4 * i + 3] = fmaf(a.w, s[4 * i + 3], k.w * vj);
-                o = fmaf(s[4 * i + 3], q.w, o);
+                o3 = fmaf(s[4 * i + 3], q.w, o3);
             }
+            float o = (o0 + o1) + (o2 + o3);
             o += __shfl_xor(o, 16, kWave);
             o += __shfl_xor(o, 32, kWave);
             if (slice == 0 && has_col) out[(static_cast<size_t>(t0 + base + tt) * heads + h) * dv + j] = o;

@@ -51,26 +51,36 @@ __device__ __forceinline__ m_u32x4 row_piece(const T* row, int k, int n, bool al
 
 constexpr int kMaxExperts = 1024;
 
-// One wavefront per token.
+// One workgroup of four wavefronts per token.  A wavefront takes the experts four at a time (all loads of the four rows
+// in flight together, then the four sums), wavefront w the groups w, w + 4, ...; the first wavefront then picks.
 template <typename T>
 __global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ x, const T* __restrict__ router,
                                                         const T* __restrict__ bias, int32_t* __restrict__ chosen,
                                                         float* __restrict__ weight, int n_tokens, int hidden, int experts,
                                                         int top) {
-    extern __shared__ float logits_s[];          // [4][experts]
+    extern __shared__ float logits_s[];          // [experts]
     const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
-    const bool live = static_cast<int>(blockIdx.x) * 4 + wave < n_tokens;
-    const int t = live ? blockIdx.x * 4 + wave : n_tokens - 1;      // a wavefront without a token repeats the last one and writes nothing
-    float* z = logits_s + wave * experts;
+    const int t = blockIdx.x;
+    float* z = logits_s;
     const T* xr = x + static_cast<size_t>(t) * hidden;
-    for (int e = 0; e < experts; ++e) {
-        const T* wr = router + static_cast<size_t>(e) * hidden;
-        float dot = 0.f;
-        for (int j = lane; j < hidden; j += kWave) dot = fmaf(to_float(xr[j]), to_float(wr[j]), dot);
-        dot = wave_sum(dot);
-        if (lane == 0) z[e] = dot + (bias ? to_float(bias[e]) : 0.f);
+    for (int e0 = wave * 4; e0 < experts; e0 += 16) {
+        float dot[4] = {0.f, 0.f, 0.f, 0.f};
+        const T* wr[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) wr[i] = router + static_cast<size_t>(min(e0 + i, experts - 1)) * hidden;
+        for (int j = lane; j < hidden; j += kWave) {
+            const float xv = to_float(xr[j]);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) dot[i] = fmaf(xv, to_float(wr[i][j]), dot[i]);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float total = wave_sum(dot[i]);
+            if (lane == 0 && e0 + i < experts) z[e0 + i] = total + (bias ? to_float(bias[e0 + i]) : 0.f);
+        }
     }
     __syncthreads();
+    if (wave != 0) return;
     // the top choices one after the other: the largest logit not yet taken, the lowest index among equals
     float first = 0.f, total = 0.f;
     for (int c = 0; c < top; ++c) {
@@ -96,15 +106,12 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ x,
         const float p = expf(best - first);      // the first choice is the largest
         total += p;
         if (lane == 0) {
-            if (live) {
-                chosen[static_cast<size_t>(t) * top + c] = best_e;
-                weight[static_cast<size_t>(t) * top + c] = p;      // divided by the total below
-            }
-            z[best_e] = -INFINITY;
+            chosen[static_cast<size_t>(t) * top + c] = best_e;
+            weight[static_cast<size_t>(t) * top + c] = p;      // divided by the total below
         }
-        __syncthreads();
+        if (lane == best_e % kWave) z[best_e] = -INFINITY;     // the lane that reads this entry takes it out
     }
-    if (lane == 0 && live) {
+    if (lane == 0) {
         const float inv = 1.0f / total;
         for (int c = 0; c < top; ++c) weight[static_cast<size_t>(t) * top + c] *= inv;
     }
@@ -178,15 +185,25 @@ __global__ __launch_bounds__(256) void moe_gate_up_kernel(const T* __restrict__ 
     m_f32x4 g[RT], u[RT];
 #pragma unroll
     for (int r = 0; r < RT; ++r) g[r] = u[r] = m_f32x4{0.f, 0.f, 0.f, 0.f};
-    for (int k0 = 0; k0 < hidden; k0 += 4 * E) {
-        const int k = k0 + lg * E;
-        const m_u32x4 a = row_piece<T>(wg, k, hidden, aligned), b = row_piece<T>(wu, k, hidden, aligned);
+    // the loads of U steps of k are issued together, so that a step waits for memory once in U
+    constexpr int U = RT >= 4 ? 2 : 4;
+    for (int k0 = 0; k0 < hidden; k0 += 4 * E * U) {
+        m_u32x4 a[U], b[U], xv[U][RT];
 #pragma unroll
-        for (int r = 0; r < RT; ++r) {
-            const m_u32x4 xv = row_piece<T>(xr[r], k, hidden, aligned);
-            g[r] = mma16<T>(a, xv, g[r]);
-            u[r] = mma16<T>(b, xv, u[r]);
+        for (int s = 0; s < U; ++s) {
+            const int k = k0 + s * 4 * E + lg * E;
+            a[s] = row_piece<T>(wg, k, hidden, aligned);
+            b[s] = row_piece<T>(wu, k, hidden, aligned);
+#pragma unroll
+            for (int r = 0; r < RT; ++r) xv[s][r] = row_piece<T>(xr[r], k, hidden, aligned);
         }
+#pragma unroll
+        for (int s = 0; s < U; ++s)
+#pragma unroll
+            for (int r = 0; r < RT; ++r) {
+                g[r] = mma16<T>(a[s], xv[s][r], g[r]);
+                u[r] = mma16<T>(b[s], xv[s][r], u[r]);
+            }
     }
     // the lane holds columns n0 + 4 lg + v of row lj of every tile of 16
 #pragma unroll
@@ -222,11 +239,20 @@ __global__ __launch_bounds__(256) void moe_down_kernel(const T* __restrict__ act
     m_f32x4 acc[RT];
 #pragma unroll
     for (int r = 0; r < RT; ++r) acc[r] = m_f32x4{0.f, 0.f, 0.f, 0.f};
-    for (int k0 = 0; k0 < ff; k0 += 4 * E) {
-        const int k = k0 + lg * E;
-        const m_u32x4 a = row_piece<T>(wd, k, ff, aligned);
+    constexpr int U = RT >= 4 ? 2 : 4;
+    for (int k0 = 0; k0 < ff; k0 += 4 * E * U) {
+        m_u32x4 a[U], av[U][RT];
 #pragma unroll
-        for (int r = 0; r < RT; ++r) acc[r] = mma16<T>(a, row_piece<T>(ar[r], k, ff, aligned), acc[r]);
+        for (int s = 0; s < U; ++s) {
+            const int k = k0 + s * 4 * E + lg * E;
+            a[s] = row_piece<T>(wd, k, ff, aligned);
+#pragma unroll
+            for (int r = 0; r < RT; ++r) av[s][r] = row_piece<T>(ar[r], k, ff, aligned);
+        }
+#pragma unroll
+        for (int s = 0; s < U; ++s)
+#pragma unroll
+            for (int r = 0; r < RT; ++r) acc[r] = mma16<T>(a[s], av[s][r], acc[r]);
     }
 #pragma unroll
     for (int r = 0; r < RT; ++r) {
@@ -264,8 +290,8 @@ extern "C" int egpt_moe_route(const void* x, const void* router, const void* bia
     if (experts > kMaxExperts) return EGPT_UNSUPPORTED_SIZE;
     if (n_tokens == 0) return EGPT_OK;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    const size_t lds = 4 * static_cast<size_t>(experts) * sizeof(float);
-    const unsigned blocks = (n_tokens + 3) / 4;
+    const size_t lds = static_cast<size_t>(experts) * sizeof(float);
+    const unsigned blocks = n_tokens;
     if (dtype == 0)
         moe_route_kernel<float><<<blocks, 256, lds, s>>>(static_cast<const float*>(x), static_cast<const float*>(router),
                                                          static_cast<const float*>(bias), chosen, weight, n_tokens, hidden,

@@ -156,8 +156,8 @@ def gated_expert(h, w, p):
 def route(h, w, p, top):
     """Chosen experts [T, top] and their weights: softmax over the chosen logits only."""
     z = h @ w[p + "router"].T + w[p + "router.b"]
-    val, idx = torch.topk(z, top, dim=-1)
-    return idx, torch.softmax(val, dim=-1), z
+    idx = torch.argsort(-z, dim=-1, stable=True)[:, :top]          # the lower index among equal logits
+    return idx, torch.softmax(torch.gather(z, -1, idx), dim=-1), z
 
 
 def expert_mixture(h, w, p, mlp):
