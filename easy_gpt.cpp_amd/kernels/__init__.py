@@ -56,6 +56,33 @@ Methods of a backend (T tokens, B requests, R rows, act = bfloat16 or float32):
         as paged_attention with key size dk and value size dv; key j <= p is read if window == 0, p - j < window or
         j < keep_first; with a sink the softmax's denominator also holds exp(sink[head])
 
+  window_attention(..., dist_bias f32[nq, far+1]|None): with a distance bias, key j of a query at position p gets
+        dist_bias[head, min(p - j, far)] added to its scaled score (a learned bias by head and distance, tabulated per
+        distance up to the one from which it no longer changes)
+
+  embed_scaled(token_ids i32[T], table act[V,H], factor, out f32[T,H])          out = table[id] * factor
+  add_layernorm(h f32[T,H], delta act[T,H]|f32[S,T,H]|None, rows i32[R]|None, weight act[H], bias act[H]|None, eps, out)
+        h += delta; out = (h - mean) / sqrt(mean((h - mean)^2) + eps) * weight + bias; with rows only those, h untouched
+  normed_pair_mean(a, b, bias_a|None, bias_b|None, weight_a, weight_b, eps, factor) -> f32[1,T,H]
+        factor * (rmsnorm(a + bias_a) * weight_a + rmsnorm(b + bias_b) * weight_b); a, b products (act or partial sums)
+  tanh_cap(x f32[...], cap)                    x = cap * tanh(x / cap) in place
+  whole_norm_store(proj, bias act[W]|None, q_out act[T,nq*dk], q_weight act[nq*dk]|None, k_weight act[nkv*dk]|None, eps,
+                   positions i32[T], coef, every, slots, k_cache, v_cache, nq, nkv, dk, dv, page_size)
+        proj rows are [nq heads of dk | nkv heads of dk | nkv heads of dv | ...]; the bias is added, queries (all heads at
+        once) and keys (likewise) are RMS-normed with a weight per value, queries multiplied by
+        1 + coef * ln(floor((p + 1) / every) + 1) (every 0: not), queries to q_out, keys and values to the pages
+  head_norm_gate(x f32[T,heads*dv], weight act[dv], eps, gate act[T,W]|f32[S,T,W], gate_offset, out act[T,heads*dv], heads, dv)
+        out = per-head rmsnorm(x) * weight * silu(gate[:, gate_offset : gate_offset + heads*dv])
+  channel_decay(low act[T,W]|f32[S,T,W], low_offset, rank, w act[C,rank], bias act[C]|None, tau) -> f32[T,C]
+        sigmoid(low[:, low_offset : low_offset + rank] w^T + bias)^(1/tau), in float32
+  decayed_state_scan(proj, act_dtype, q_offset, k_offset, v_offset, q_scale, decay f32[T,heads*dk], states f32[slots,heads,dk,dv],
+                     slots i32[B], fresh bool[B]|None, q_start i32[B], q_len i32[B], heads, dk, dv) -> f32[T,heads*dv]
+        per request and head, token by token: S = diag(decay_t) S + k_t v_t^T, o_t = S^T (q_t * q_scale); S is read from and
+        written to states[slots[b]] (fresh[b]: it starts at zero); q, k, v are columns of the product rows
+  expert_mixture(x act[T,H], router act[E,H], router_bias act[E]|None, w_gate_up act[E,2F,H], w_down act[E,H,F], top) -> f32[T,H]
+        float32 logits x router^T + bias, the `top` largest (lowest index among equals), softmax over those; the weighted
+        sum of down_e(silu(gate_e x) * (up_e x)) over the chosen experts e, added in the order of the choices
+
 Beside these, a backend has fused variants that fold neighbouring operations into one kernel.  They are part of
 the contract too (`KernelBackend` below): each returns None (False for the decode attention) where it does not
 cover a case, and the caller then takes the unfused way.
