@@ -412,10 +412,10 @@ def nebanex_config(width, heads, kv_heads, hd, s_heads, s_dim, s_vdim, experts, 
     layer = {"type": "parallel",
              "mixer": {"left": {"heads": heads, "kv_heads": kv_heads, "dim": hd, "vdim": hd, "scale": hd ** -0.5, "bias_max": 512,
                                 "q_temp": {"coef": 0.1, "every": 1024}},
-                       "right": {"heads": s_heads, "dim": s_dim, "vdim": s_vdim, "tau": 16.0}},
+                       "right": {"heads": s_heads, "dim": s_dim, "vdim": s_vdim, "tau": 8.0}},
              "mlp": {"kind": "moe", "router": {"experts": experts, "top": top}, "expert": {"ff": ff}, "shared": {"ff": shared}}}
     return {"architecture": "Nebanex", "vocab": DESIGN_VOCAB, "width": width, "norm": {"eps": 1e-6}, "embedding": {"scale": 1.0},
-            "logit_softcap": 30.0, "layers": [layer] * DESIGN_LAYERS}
+            "logit_softcap": 50.0, "layers": [layer] * DESIGN_LAYERS}
 
 
 def design_models(design):

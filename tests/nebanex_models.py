@@ -15,7 +15,7 @@ import torch
 from easy_gpt.cpp_amd.weights import write_safetensors
 
 
-def left(heads, kv_heads, dim, vdim, scale, bias_max, coef=0.3, every=16):
+def left(heads, kv_heads, dim, vdim, scale, bias_max, coef=0.4, every=16):
     m = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": scale, "bias_max": bias_max}
     if every:
         m["q_temp"] = {"coef": coef, "every": every}
@@ -59,14 +59,14 @@ CONFIG_B = {
 }
 # multiples of 16, so that the matrix-core attention runs; every expert chosen; keys of 64 and 160 in the state
 CONFIG_C = {
-    "architecture": "Nebanex", "vocab": 411, "width": 128, "norm": {"eps": 1e-6}, "embedding": {"scale": 12.0},
-    "logit_softcap": 30.0,
+    "architecture": "Nebanex", "vocab": 411, "width": 128, "norm": {"eps": 1e-6}, "embedding": {"scale": 10.0},
+    "logit_softcap": 25.0,
     "layers": [
-        layer(left(4, 1, 64, 32, 0.125, 50, 0.3, 64), right(2, 64, 80, 4.0), moe(8, 8, 64, 32)),
-        layer(left(8, 2, 32, 64, 0.18, 100, 0.3, 128), right(1, 160, 64, 16.0), moe(16, 4, 32, 96)),
+        layer(left(4, 1, 64, 32, 0.11, 50, 0.35, 64), right(2, 64, 80, 4.0), moe(8, 8, 64, 32)),
+        layer(left(8, 2, 32, 64, 0.18, 100, 0.2, 96), right(1, 160, 64, 12.0), moe(16, 4, 32, 96)),
     ],
 }
-CONFIGS = {"A": (CONFIG_A, 5, 8, 5), "B": (CONFIG_B, 6, 6, 3), "C": (CONFIG_C, 7, 16, 16)}      # config, seed, bias rows, decay rank
+CONFIGS = {"A": (CONFIG_A, 5, 8, 5), "B": (CONFIG_B, 6, 6, 3), "C": (CONFIG_C, 7, 12, 8)}      # config, seed, bias rows, decay rank
 
 
 def draw_weights(cfg: dict, seed: int, bias_rows: int = 8, rank: int = 5, sharp: float = 3.0) -> dict[str, torch.Tensor]:

@@ -27,7 +27,7 @@ CONFIG_D = {
     "architecture": "Nebanex", "vocab": 523, "width": 256, "norm": {"eps": 1e-5}, "embedding": {"scale": 16.0},
     "logit_softcap": 20.0,
     "layers": [
-        NM.layer(NM.left(8, 2, 64, 64, 0.125, 300, 0.3, 128), NM.right(2, 128, 128, 16.0), NM.moe(16, 4, 128, 256)),
+        NM.layer(NM.left(8, 2, 64, 64, 0.12, 300, 0.2, 96), NM.right(2, 128, 128, 12.0), NM.moe(16, 4, 128, 256)),
         NM.layer(NM.left(2, 1, 128, 128, 0.09, 64, 0.1, 100), NM.right(4, 32, 64, 8.0), NM.moe(4, 2, 64, None)),
     ],
 }

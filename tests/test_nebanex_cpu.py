@@ -133,10 +133,9 @@ def test_a_missing_tensor_is_named(tmp_path, emulated):
 
 # ----------------------------------------------------------------------------- pins of the plain mechanisms
 def test_distance_buckets_are_exact_up_close_and_logarithmic_beyond():
-    assert [P.distance_bucket(n, 16, 120) for n in range(9)] == [0, 1, 2, 3, 4, 5, 6, 7, 8]
-    # 8 * 15^(k/8) is where row 8 + k starts: 8, 11.2, 15.7, 22.1, 31.0, 43.5, 61.0, 85.5
-    assert [P.distance_bucket(n, 16, 120) for n in (11, 12, 15, 16, 22, 23, 30, 31, 43, 44, 60, 61, 85, 86, 119, 120, 5000)] == \
-        [8, 9, 9, 10, 10, 11, 11, 12, 12, 13, 13, 14, 14, 15, 15, 15, 15]
+    assert [P.distance_bucket(n, 10, 70) for n in range(6)] == [0, 1, 2, 3, 4, 5]
+    # 5 * 14^(k/5) is where row 5 + k starts: 5, 8.5, 14.4, 24.4, 41.3, 70
+    assert [P.distance_bucket(n, 10, 70) for n in (8, 9, 14, 15, 24, 25, 41, 42, 69, 70, 5000)] == [5, 6, 6, 7, 7, 8, 8, 9, 9, 9, 9]
     for rows, far in [(8, 20), (6, 9), (16, 50), (32, 300), (4, 3)]:
         b = [P.distance_bucket(n, rows, far) for n in range(far + 40)]
         assert b[: rows // 2] == list(range(rows // 2)) and b == sorted(b) and max(b) == rows - 1 and b[far] == rows - 1
