@@ -44,53 +44,53 @@ __global__ __launch_bounds__(256) void channel_decay_kernel(ProductView<T> low, 
     }
 }
 
-constexpr int kScanTokens = 16;     // tokens staged in LDS at a time
-constexpr int kScanCols = 64;       // value channels per workgroup
+constexpr int kScanTokens = 8;      // tokens staged in LDS at a time
+constexpr int kScanCols = 64;       // value channels per workgroup: a lane is a column of the state
 
-// One workgroup of four wavefronts per (request, head, 64 value channels).  A wavefront takes 16 value channels; its
-// lanes are 4 slices of the key channels times 16 value channels, a lane keeps DKR key channels of one column of the
-// state in registers, and the four slices' parts of o_t are added across the lanes in a fixed order.  Queries, keys,
-// decays and values of kScanTokens tokens are staged in LDS (a slice's rows padded apart so that the four slices
-// read different banks).
-template <typename T, int DKR>
-__global__ __launch_bounds__(256) void decayed_state_scan_kernel(
+// One workgroup of NS wavefronts per (request, head, 64 value channels).  A lane is one column of the state; wavefront w
+// keeps the DKR key channels w * DKR .. of that column in registers (dk <= NS * DKR), so a token costs a lane 3 DKR
+// multiply-adds, and the queries, keys and decays that a wavefront needs are the same for all its lanes: it reads them
+// from LDS at one address.  The wavefronts' parts of o_t go through LDS and are added in the order of the wavefronts,
+// a batch of kScanTokens tokens at a time.  The batch's queries, keys, decays and values are staged in LDS, the next
+// batch's loads in flight in registers meanwhile.
+template <typename T, int DKR, int NS>
+__global__ __launch_bounds__(64 * NS) void decayed_state_scan_kernel(
     ProductView<T> proj, int proj_width, int q_off, int k_off, int v_off, float q_scale, const float* __restrict__ decay,
     float* __restrict__ states, const int32_t* __restrict__ slots, const unsigned char* __restrict__ fresh,
     const int32_t* __restrict__ q_start, const int32_t* __restrict__ q_len, float* __restrict__ out, int heads, int dk, int dv) {
-    constexpr int ROW = DKR + 4;                 // a slice's row in LDS
-    constexpr int TOK = 4 * ROW;                 // a token's q (or k, or decay) in LDS
-    __shared__ __attribute__((aligned(16))) float q_s[kScanTokens * TOK];
-    __shared__ __attribute__((aligned(16))) float k_s[kScanTokens * TOK];
-    __shared__ __attribute__((aligned(16))) float a_s[kScanTokens * TOK];
+    constexpr int THREADS = 64 * NS;
+    constexpr int DKP = NS * DKR;                             // key channels with padding
+    constexpr int QKA = kScanTokens * DKP / THREADS;          // values of q (or k, or decays) of a batch per thread
+    constexpr int VL = kScanTokens * kScanCols / THREADS;     // values of v, and outputs, of a batch per thread
+    static_assert(QKA * THREADS == kScanTokens * DKP && VL * THREADS == kScanTokens * kScanCols && VL >= 1, "a batch divides evenly");
+    __shared__ __attribute__((aligned(16))) float q_s[kScanTokens * DKP];
+    __shared__ __attribute__((aligned(16))) float k_s[kScanTokens * DKP];
+    __shared__ __attribute__((aligned(16))) float a_s[kScanTokens * DKP];
     __shared__ float v_s[kScanTokens * kScanCols];
+    __shared__ float part_s[kScanTokens * NS * kScanCols];
     const int b = blockIdx.x, h = blockIdx.y, col0 = blockIdx.z * kScanCols;
     const int n = q_len[b];
     if (n <= 0) return;
     const int t0 = q_start[b];
     const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
-    const int slice = lane / 16, col = wave * 16 + lane % 16;
-    const int j = col0 + col;
+    const int j = col0 + lane;
     const bool has_col = j < dv;
     float* state = states + (static_cast<size_t>(slots[b]) * heads + h) * dk * dv;
     float s[DKR];
     const bool start_anew = fresh != nullptr && fresh[b] != 0;
 #pragma unroll
     for (int i = 0; i < DKR; ++i) {
-        const int r = slice * DKR + i;
+        const int r = wave * DKR + i;
         s[i] = (!start_anew && has_col && r < dk) ? state[static_cast<size_t>(r) * dv + j] : 0.f;
     }
     const int channels = heads * dk;
-    // The next tokens' queries, keys, decays and values travel through registers: their loads are issued before this
-    // batch of tokens is computed and stored to LDS behind it, so that a batch waits for memory once, not once per
-    // array, and not at all while the recurrence runs long.
-    constexpr int QKA = kScanTokens * 4 * DKR / 256, VL = kScanTokens * kScanCols / 256;
     float rq[QKA], rk[QKA], ra[QKA], rv[VL];
     auto fetch = [&](int base) {
         const int count = min(kScanTokens, n - base);
 #pragma unroll
         for (int u = 0; u < QKA; ++u) {
-            const int idx = tid + u * 256;
-            const int tt = idx / (4 * DKR), r = idx % (4 * DKR);
+            const int idx = tid + u * THREADS;
+            const int tt = idx / DKP, r = idx % DKP;
             rq[u] = rk[u] = ra[u] = 0.f;
             if (tt < count && r < dk) {
                 const size_t row = static_cast<size_t>(t0 + base + tt);
@@ -101,7 +101,7 @@ __global__ __launch_bounds__(256) void decayed_state_scan_kernel(
         }
 #pragma unroll
         for (int u = 0; u < VL; ++u) {
-            const int idx = tid + u * 256;
+            const int idx = tid + u * THREADS;
             const int tt = idx / kScanCols, c = idx % kScanCols;
             rv[u] = 0.f;
             if (tt < count && col0 + c < dv)
@@ -111,25 +111,22 @@ __global__ __launch_bounds__(256) void decayed_state_scan_kernel(
     fetch(0);
     for (int base = 0; base < n; base += kScanTokens) {
         const int count = min(kScanTokens, n - base);
-        __syncthreads();                          // the tokens before are read
+        __syncthreads();                          // the batch before is read, its parts are added
 #pragma unroll
         for (int u = 0; u < QKA; ++u) {
-            const int idx = tid + u * 256;
-            const int tt = idx / (4 * DKR), r = idx % (4 * DKR);
-            const int at = tt * TOK + (r / DKR) * ROW + r % DKR;
-            q_s[at] = rq[u];
-            k_s[at] = rk[u];
-            a_s[at] = ra[u];
+            q_s[tid + u * THREADS] = rq[u];
+            k_s[tid + u * THREADS] = rk[u];
+            a_s[tid + u * THREADS] = ra[u];
         }
 #pragma unroll
-        for (int u = 0; u < VL; ++u) v_s[tid + u * 256] = rv[u];
+        for (int u = 0; u < VL; ++u) v_s[tid + u * THREADS] = rv[u];
         __syncthreads();
         if (base + kScanTokens < n) fetch(base + kScanTokens);
         for (int tt = 0; tt < count; ++tt) {
-            const float vj = v_s[tt * kScanCols + col];
-            const float4* a4 = reinterpret_cast<const float4*>(a_s + tt * TOK + slice * ROW);
-            const float4* k4 = reinterpret_cast<const float4*>(k_s + tt * TOK + slice * ROW);
-            const float4* q4 = reinterpret_cast<const float4*>(q_s + tt * TOK + slice * ROW);
+            const float vj = v_s[tt * kScanCols + lane];
+            const float4* a4 = reinterpret_cast<const float4*>(a_s + tt * DKP + wave * DKR);
+            const float4* k4 = reinterpret_cast<const float4*>(k_s + tt * DKP + wave * DKR);
+            const float4* q4 = reinterpret_cast<const float4*>(q_s + tt * DKP + wave * DKR);
             float o0 = 0.f, o1 = 0.f, o2 = 0.f, o3 = 0.f;       // four sums, so that no addition waits for the one before
 #pragma unroll
             for (int i = 0; i < DKR / 4; ++i) {
@@ -143,16 +140,25 @@ __global__ __launch_bounds__(256) void decayed_state_scan_kernel(
                 s[4 * i + 3] = fmaf(a.w, s[4 * i + 3], k.w * vj);
                 o3 = fmaf(s[4 * i + 3], q.w, o3);
             }
-            float o = (o0 + o1) + (o2 + o3);
-            o += __shfl_xor(o, 16, kWave);
-            o += __shfl_xor(o, 32, kWave);
-            if (slice == 0 && has_col) out[(static_cast<size_t>(t0 + base + tt) * heads + h) * dv + j] = o;
+            part_s[(tt * NS + wave) * kScanCols + lane] = (o0 + o1) + (o2 + o3);
+        }
+        __syncthreads();
+#pragma unroll
+        for (int u = 0; u < VL; ++u) {
+            const int idx = tid + u * THREADS;
+            const int tt = idx / kScanCols, c = idx % kScanCols;
+            if (tt < count && col0 + c < dv) {
+                float o = 0.f;
+#pragma unroll
+                for (int w = 0; w < NS; ++w) o += part_s[(tt * NS + w) * kScanCols + c];
+                out[(static_cast<size_t>(t0 + base + tt) * heads + h) * dv + col0 + c] = o;
+            }
         }
     }
     if (has_col) {
 #pragma unroll
         for (int i = 0; i < DKR; ++i) {
-            const int r = slice * DKR + i;
+            const int r = wave * DKR + i;
             if (r < dk) state[static_cast<size_t>(r) * dv + j] = s[i];
         }
     }
@@ -190,13 +196,13 @@ static int launch_scan(const void* proj, int n_splits, int proj_width, int q_off
                        int dv, hipStream_t s) {
     const ProductView<T> view = scan_view<T>(proj, n_splits, static_cast<size_t>(n_tokens) * proj_width);
     dim3 grid(n_seqs, heads, (dv + kScanCols - 1) / kScanCols);
-#define EGPT_SCAN(DKR_)                                                                                                   \
-    decayed_state_scan_kernel<T, DKR_><<<grid, 256, 0, s>>>(view, proj_width, q_off, k_off, v_off, q_scale, decay, states, \
-                                                            slots, fresh, q_start, q_len, out, heads, dk, dv)
-    if (dk <= 32) EGPT_SCAN(8);
-    else if (dk <= 64) EGPT_SCAN(16);
-    else if (dk <= 128) EGPT_SCAN(32);
-    else EGPT_SCAN(64);
+#define EGPT_SCAN(DKR_, NS_)                                                                                            \
+    decayed_state_scan_kernel<T, DKR_, NS_><<<grid, 64 * NS_, 0, s>>>(view, proj_width, q_off, k_off, v_off, q_scale, decay, \
+                                                                      states, slots, fresh, q_start, q_len, out, heads, dk, dv)
+    if (dk <= 32) EGPT_SCAN(8, 4);
+    else if (dk <= 64) EGPT_SCAN(8, 8);
+    else if (dk <= 128) EGPT_SCAN(16, 8);
+    else EGPT_SCAN(32, 8);
 #undef EGPT_SCAN
     return EGPT_OK;
 }
