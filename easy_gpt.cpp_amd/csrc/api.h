@@ -191,8 +191,9 @@ int egpt_whole_norm_store(const void* proj, int n_splits, int row_width, const v
                           const void* q_weight, const void* k_weight, float eps, const int32_t* positions, float coef,
                           int every, const int32_t* slots, void* k_cache, void* v_cache, int n_tokens, int nq, int nkv,
                           int dk, int dv, int page_size, int dtype, void* stream);
-// out = per-head rmsnorm(x float32 [n_tokens][heads][dv]) * weight[dv] * silu(gate columns gate_off.. of a product row)
-int egpt_head_norm_gate(const float* x, const void* weight, float eps, const void* gate, int gate_splits, int gate_width,
+// out = per-head rmsnorm(x) * weight[dv] * silu(gate columns gate_off.. of a product row); x float32 [n_tokens][heads][dv]
+// (x_splits 0) or partial sums [x_splits][n_tokens][heads][dv]
+int egpt_head_norm_gate(const float* x, int x_splits, const void* weight, float eps, const void* gate, int gate_splits, int gate_width,
                         int gate_off, void* out, int n_tokens, int heads, int dv, int dtype, void* stream);
 // ---- linear_recurrence.hip: a matrix state per head that decays per key channel
 // decay[t][c] = sigmoid(z)^(1 / tau), z = bias[c] + sum_r w[c][r] * low[t][r]; low: columns low_off.. of a product row.
@@ -200,7 +201,9 @@ int egpt_channel_decay(const void* low, int low_splits, int low_width, int low_o
                        float tau, float* decay, int n_tokens, int channels, int dtype, void* stream);
 // S <- diag(decay_t) S + k_t v_t^T, o_t = S^T (q_t * q_scale), token by token for every request of the step; the state
 // float32 [slots][heads][dk][dv] is read from and written to states[slot[b]] (fresh[b] != 0: it starts at zero).
-// q, k, v: columns q_off, k_off, v_off of a product row of proj_width values.  out float32 [n_tokens][heads][dv].
+// q, k, v: columns q_off, k_off, v_off of a product row of proj_width values.  out float32 [egpt_scan_key_splits(dk)][n_tokens][heads][dv]:
+// partial sums over ranges of the key channels, for the consumer to add.
+int egpt_scan_key_splits(int dk);
 int egpt_decayed_state_scan(const void* proj, int n_splits, int proj_width, int q_off, int k_off, int v_off, float q_scale,
                             const float* decay, float* states, const int32_t* slots, const unsigned char* fresh,
                             const int32_t* q_start, const int32_t* q_len, int n_seqs, int n_tokens, float* out, int heads,

@@ -271,20 +271,23 @@ __global__ __launch_bounds__(256) void whole_norm_store_kernel(
 }
 
 // out[t][h * dv + d] = x[t][h * dv + d] / rms(x[t][h * dv ..]) * weight[d] * silu(g[t][gate_off + h * dv + d]): the
-// RMS norm of every head's float32 output with a weight that the heads share, and a SiLU gate from columns of a
+// RMS norm of every head's float32 output (one tensor, or partial sums that are added here) with a weight that the heads share, and a SiLU gate from columns of a
 // product row.  One wavefront per (token, head).
 template <typename T>
-__global__ __launch_bounds__(kWave) void head_norm_gate_kernel(const float* __restrict__ x, const T* __restrict__ weight,
+__global__ __launch_bounds__(kWave) void head_norm_gate_kernel(ProductView<float> x, const T* __restrict__ weight,
                                                                float eps, ProductView<T> g, int gate_width, int gate_off,
                                                                T* __restrict__ out, int heads, int dv) {
     const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
-    const float* xr = x + (static_cast<size_t>(t) * heads + h) * dv;
+    const size_t xr = (static_cast<size_t>(t) * heads + h) * dv;
     float ss = 0.f;
-    for (int d = lane; d < dv; d += kWave) ss = fmaf(xr[d], xr[d], ss);
+    for (int d = lane; d < dv; d += kWave) {
+        const float v = x.at(xr + d);
+        ss = fmaf(v, v, ss);
+    }
     const float inv = inv_rms(wave_sum(ss), 1.0f / static_cast<float>(dv), eps);
     for (int d = lane; d < dv; d += kWave) {
         const float gate = g.at(static_cast<size_t>(t) * gate_width + gate_off + h * dv + d);
-        const float y = xr[d] * inv * to_float(weight[d]) * (gate / (1.0f + expf(-gate)));
+        const float y = x.at(xr + d) * inv * to_float(weight[d]) * (gate / (1.0f + expf(-gate)));
         out[(static_cast<size_t>(t) * heads + h) * dv + d] = from_float<T>(y);
     }
 }
@@ -439,10 +442,10 @@ extern "C" int egpt_whole_norm_store(const void* proj, int n_splits, int row_wid
     return EGPT_OK;
 }
 
-extern "C" int egpt_head_norm_gate(const float* x, const void* weight, float eps, const void* gate, int gate_splits,
+extern "C" int egpt_head_norm_gate(const float* x, int x_splits, const void* weight, float eps, const void* gate, int gate_splits,
                                    int gate_width, int gate_off, void* out, int n_tokens, int heads, int dv, int dtype,
                                    void* stream) {
-    if (!x || !weight || !gate || !out || n_tokens < 0 || heads <= 0 || dv <= 0 || gate_splits < 0 || gate_off < 0 ||
+    if (!x || x_splits < 0 || !weight || !gate || !out || n_tokens < 0 || heads <= 0 || dv <= 0 || gate_splits < 0 || gate_off < 0 ||
         gate_off + heads * dv > gate_width || (dtype != 0 && dtype != 1))
         return EGPT_BAD_ARGUMENT;
     if (heads > 65535) return EGPT_UNSUPPORTED_SIZE;
@@ -450,12 +453,18 @@ extern "C" int egpt_head_norm_gate(const float* x, const void* weight, float eps
     hipStream_t s = static_cast<hipStream_t>(stream);
     const size_t stride = static_cast<size_t>(n_tokens) * gate_width;
     dim3 grid(n_tokens, heads);
+    // x float32 [n_tokens][heads * dv] (x_splits 0) or partial sums [x_splits][n_tokens][heads * dv]
+    ProductView<float> xv;
+    xv.whole = x_splits == 0 ? x : nullptr;
+    xv.partial = x_splits > 0 ? x : nullptr;
+    xv.n_splits = x_splits;
+    xv.split_stride = static_cast<size_t>(n_tokens) * heads * dv;
     if (dtype == 0)
-        head_norm_gate_kernel<float><<<grid, kWave, 0, s>>>(x, static_cast<const float*>(weight), eps,
+        head_norm_gate_kernel<float><<<grid, kWave, 0, s>>>(xv, static_cast<const float*>(weight), eps,
                                                             view_of<float>(gate, gate_splits, stride), gate_width, gate_off,
                                                             static_cast<float*>(out), heads, dv);
     else
-        head_norm_gate_kernel<bf16_t><<<grid, kWave, 0, s>>>(x, static_cast<const bf16_t*>(weight), eps,
+        head_norm_gate_kernel<bf16_t><<<grid, kWave, 0, s>>>(xv, static_cast<const bf16_t*>(weight), eps,
                                                              view_of<bf16_t>(gate, gate_splits, stride), gate_width, gate_off,
                                                              static_cast<bf16_t*>(out), heads, dv);
     EGPT_CHECK_LAUNCH();

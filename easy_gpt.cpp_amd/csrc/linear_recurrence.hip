@@ -44,31 +44,36 @@ __global__ __launch_bounds__(256) void channel_decay_kernel(ProductView<T> low, 
     }
 }
 
-constexpr int kScanTokens = 8;      // tokens staged in LDS at a time
+constexpr int kScanTokens = 32;     // tokens staged in LDS at a time
 constexpr int kScanCols = 64;       // value channels per workgroup: a lane is a column of the state
+constexpr int kScanKeys = 16;       // key channels per workgroup
+constexpr int kScanWaves = 4;       // wavefronts per workgroup, kScanKeys / kScanWaves key channels each
 
-// One workgroup of NS wavefronts per (request, head, 64 value channels).  A lane is one column of the state; wavefront w
-// keeps the DKR key channels w * DKR .. of that column in registers (dk <= NS * DKR), so a token costs a lane 3 DKR
-// multiply-adds, and the queries, keys and decays that a wavefront needs are the same for all its lanes: it reads them
-// from LDS at one address.  The wavefronts' parts of o_t go through LDS and are added in the order of the wavefronts,
-// a batch of kScanTokens tokens at a time.  The batch's queries, keys, decays and values are staged in LDS, the next
-// batch's loads in flight in registers meanwhile.
-template <typename T, int DKR, int NS>
-__global__ __launch_bounds__(64 * NS) void decayed_state_scan_kernel(
+// The recurrence has no term that mixes two key channels but the sum o_t = sum_r S[r][:] q[r], so the key channels are
+// dealt over workgroups: one workgroup of four wavefronts per (request, head, 64 value channels, 16 key channels), whose
+// part of o_t goes to out[split] (float32 [splits][tokens][heads * dv]) for the consumer to add in the order of the
+// splits.  A lane is one column of the state; wavefront w keeps four of the workgroup's key channels of that column in
+// registers.  The queries, keys and decays that a wavefront needs are the same for all its lanes (one address in LDS);
+// what bounds a token is what LDS returns for them (every lane gets its copy), which is why a workgroup takes few key
+// channels.  The wavefronts' parts go through LDS and are added in the order of the wavefronts, a batch of kScanTokens
+// tokens at a time; the batch's operands are staged in LDS, the next batch's loads in flight in registers meanwhile.
+template <typename T>
+__global__ __launch_bounds__(64 * kScanWaves) void decayed_state_scan_kernel(
     ProductView<T> proj, int proj_width, int q_off, int k_off, int v_off, float q_scale, const float* __restrict__ decay,
     float* __restrict__ states, const int32_t* __restrict__ slots, const unsigned char* __restrict__ fresh,
-    const int32_t* __restrict__ q_start, const int32_t* __restrict__ q_len, float* __restrict__ out, int heads, int dk, int dv) {
-    constexpr int THREADS = 64 * NS;
-    constexpr int DKP = NS * DKR;                             // key channels with padding
+    const int32_t* __restrict__ q_start, const int32_t* __restrict__ q_len, float* __restrict__ out, int n_tokens, int heads,
+    int dk, int dv, int key_splits) {
+    constexpr int NS = kScanWaves, DKR = kScanKeys / kScanWaves, THREADS = 64 * NS, DKP = kScanKeys;
     constexpr int QKA = kScanTokens * DKP / THREADS;          // values of q (or k, or decays) of a batch per thread
     constexpr int VL = kScanTokens * kScanCols / THREADS;     // values of v, and outputs, of a batch per thread
-    static_assert(QKA * THREADS == kScanTokens * DKP && VL * THREADS == kScanTokens * kScanCols && VL >= 1, "a batch divides evenly");
+    static_assert(DKR == 4 && QKA * THREADS == kScanTokens * DKP && VL * THREADS == kScanTokens * kScanCols, "a batch divides evenly");
     __shared__ __attribute__((aligned(16))) float q_s[kScanTokens * DKP];
     __shared__ __attribute__((aligned(16))) float k_s[kScanTokens * DKP];
     __shared__ __attribute__((aligned(16))) float a_s[kScanTokens * DKP];
     __shared__ float v_s[kScanTokens * kScanCols];
     __shared__ float part_s[kScanTokens * NS * kScanCols];
-    const int b = blockIdx.x, h = blockIdx.y, col0 = blockIdx.z * kScanCols;
+    const int b = blockIdx.x, h = blockIdx.y;
+    const int split = blockIdx.z % key_splits, col0 = (blockIdx.z / key_splits) * kScanCols, key0 = split * kScanKeys;
     const int n = q_len[b];
     if (n <= 0) return;
     const int t0 = q_start[b];
@@ -76,11 +81,12 @@ __global__ __launch_bounds__(64 * NS) void decayed_state_scan_kernel(
     const int j = col0 + lane;
     const bool has_col = j < dv;
     float* state = states + (static_cast<size_t>(slots[b]) * heads + h) * dk * dv;
+    float* o_split = out + static_cast<size_t>(split) * n_tokens * heads * dv;
     float s[DKR];
     const bool start_anew = fresh != nullptr && fresh[b] != 0;
 #pragma unroll
     for (int i = 0; i < DKR; ++i) {
-        const int r = wave * DKR + i;
+        const int r = key0 + wave * DKR + i;
         s[i] = (!start_anew && has_col && r < dk) ? state[static_cast<size_t>(r) * dv + j] : 0.f;
     }
     const int channels = heads * dk;
@@ -90,7 +96,7 @@ __global__ __launch_bounds__(64 * NS) void decayed_state_scan_kernel(
 #pragma unroll
         for (int u = 0; u < QKA; ++u) {
             const int idx = tid + u * THREADS;
-            const int tt = idx / DKP, r = idx % DKP;
+            const int tt = idx / DKP, r = key0 + idx % DKP;
             rq[u] = rk[u] = ra[u] = 0.f;
             if (tt < count && r < dk) {
                 const size_t row = static_cast<size_t>(t0 + base + tt);
@@ -124,23 +130,14 @@ __global__ __launch_bounds__(64 * NS) void decayed_state_scan_kernel(
         if (base + kScanTokens < n) fetch(base + kScanTokens);
         for (int tt = 0; tt < count; ++tt) {
             const float vj = v_s[tt * kScanCols + lane];
-            const float4* a4 = reinterpret_cast<const float4*>(a_s + tt * DKP + wave * DKR);
-            const float4* k4 = reinterpret_cast<const float4*>(k_s + tt * DKP + wave * DKR);
-            const float4* q4 = reinterpret_cast<const float4*>(q_s + tt * DKP + wave * DKR);
-            float o0 = 0.f, o1 = 0.f, o2 = 0.f, o3 = 0.f;       // four sums, so that no addition waits for the one before
-#pragma unroll
-            for (int i = 0; i < DKR / 4; ++i) {
-                const float4 a = a4[i], k = k4[i], q = q4[i];
-                s[4 * i] = fmaf(a.x, s[4 * i], k.x * vj);
-                o0 = fmaf(s[4 * i], q.x, o0);
-                s[4 * i + 1] = fmaf(a.y, s[4 * i + 1], k.y * vj);
-                o1 = fmaf(s[4 * i + 1], q.y, o1);
-                s[4 * i + 2] = fmaf(a.z, s[4 * i + 2], k.z * vj);
-                o2 = fmaf(s[4 * i + 2], q.z, o2);
-                s[4 * i + 3] = fmaf(a.w, s[4 * i + 3], k.w * vj);
-                o3 = fmaf(s[4 * i + 3], q.w, o3);
-            }
-            part_s[(tt * NS + wave) * kScanCols + lane] = (o0 + o1) + (o2 + o3);
+            const float4 a = *reinterpret_cast<const float4*>(a_s + tt * DKP + wave * DKR);
+            const float4 k = *reinterpret_cast<const float4*>(k_s + tt * DKP + wave * DKR);
+            const float4 q = *reinterpret_cast<const float4*>(q_s + tt * DKP + wave * DKR);
+            s[0] = fmaf(a.x, s[0], k.x * vj);
+            s[1] = fmaf(a.y, s[1], k.y * vj);
+            s[2] = fmaf(a.z, s[2], k.z * vj);
+            s[3] = fmaf(a.w, s[3], k.w * vj);
+            part_s[(tt * NS + wave) * kScanCols + lane] = (s[0] * q.x + s[1] * q.y) + (s[2] * q.z + s[3] * q.w);
         }
         __syncthreads();
 #pragma unroll
@@ -151,14 +148,14 @@ __global__ __launch_bounds__(64 * NS) void decayed_state_scan_kernel(
                 float o = 0.f;
 #pragma unroll
                 for (int w = 0; w < NS; ++w) o += part_s[(tt * NS + w) * kScanCols + c];
-                out[(static_cast<size_t>(t0 + base + tt) * heads + h) * dv + col0 + c] = o;
+                o_split[(static_cast<size_t>(t0 + base + tt) * heads + h) * dv + col0 + c] = o;
             }
         }
     }
     if (has_col) {
 #pragma unroll
         for (int i = 0; i < DKR; ++i) {
-            const int r = wave * DKR + i;
+            const int r = key0 + wave * DKR + i;
             if (r < dk) state[static_cast<size_t>(r) * dv + j] = s[i];
         }
     }
@@ -195,17 +192,14 @@ static int launch_scan(const void* proj, int n_splits, int proj_width, int q_off
                        const int32_t* q_start, const int32_t* q_len, int n_seqs, int n_tokens, float* out, int heads, int dk,
                        int dv, hipStream_t s) {
     const ProductView<T> view = scan_view<T>(proj, n_splits, static_cast<size_t>(n_tokens) * proj_width);
-    dim3 grid(n_seqs, heads, (dv + kScanCols - 1) / kScanCols);
-#define EGPT_SCAN(DKR_, NS_)                                                                                            \
-    decayed_state_scan_kernel<T, DKR_, NS_><<<grid, 64 * NS_, 0, s>>>(view, proj_width, q_off, k_off, v_off, q_scale, decay, \
-                                                                      states, slots, fresh, q_start, q_len, out, heads, dk, dv)
-    if (dk <= 32) EGPT_SCAN(8, 4);
-    else if (dk <= 64) EGPT_SCAN(8, 8);
-    else if (dk <= 128) EGPT_SCAN(16, 8);
-    else EGPT_SCAN(32, 8);
-#undef EGPT_SCAN
+    const int key_splits = (dk + kScanKeys - 1) / kScanKeys;
+    dim3 grid(n_seqs, heads, (dv + kScanCols - 1) / kScanCols * key_splits);
+    decayed_state_scan_kernel<T><<<grid, 64 * kScanWaves, 0, s>>>(view, proj_width, q_off, k_off, v_off, q_scale, decay, states, slots,
+                                                                  fresh, q_start, q_len, out, n_tokens, heads, dk, dv, key_splits);
     return EGPT_OK;
 }
+
+extern "C" int egpt_scan_key_splits(int dk) { return dk > 0 ? (dk + kScanKeys - 1) / kScanKeys : 0; }
 
 extern "C" int egpt_decayed_state_scan(const void* proj, int n_splits, int proj_width, int q_off, int k_off, int v_off,
                                        float q_scale, const float* decay, float* states, const int32_t* slots,
@@ -216,7 +210,8 @@ extern "C" int egpt_decayed_state_scan(const void* proj, int n_splits, int proj_
         return EGPT_BAD_ARGUMENT;
     if (q_off + heads * dk > proj_width || k_off + heads * dk > proj_width || v_off + heads * dv > proj_width)
         return EGPT_BAD_ARGUMENT;
-    if (dk > 256 || heads > 65535 || (dv + kScanCols - 1) / kScanCols > 65535) return EGPT_UNSUPPORTED_SIZE;
+    if (heads > 65535 || static_cast<long long>((dv + kScanCols - 1) / kScanCols) * ((dk + kScanKeys - 1) / kScanKeys) > 65535)
+        return EGPT_UNSUPPORTED_SIZE;
     if (n_tokens == 0) return EGPT_OK;
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (dtype == 0)

@@ -71,14 +71,15 @@ Methods of a backend (T tokens, B requests, R rows, act = bfloat16 or float32):
         proj rows are [nq heads of dk | nkv heads of dk | nkv heads of dv | ...]; the bias is added, queries (all heads at
         once) and keys (likewise) are RMS-normed with a weight per value, queries multiplied by
         1 + coef * ln(floor((p + 1) / every) + 1) (every 0: not), queries to q_out, keys and values to the pages
-  head_norm_gate(x f32[T,heads*dv], weight act[dv], eps, gate act[T,W]|f32[S,T,W], gate_offset, out act[T,heads*dv], heads, dv)
+  head_norm_gate(x f32[T,heads*dv]|f32[S,T,heads*dv], weight act[dv], eps, gate act[T,W]|f32[S,T,W], gate_offset, out act[T,heads*dv], heads, dv)
         out = per-head rmsnorm(x) * weight * silu(gate[:, gate_offset : gate_offset + heads*dv])
   channel_decay(low act[T,W]|f32[S,T,W], low_offset, rank, w act[C,rank], bias act[C]|None, tau) -> f32[T,C]
         sigmoid(low[:, low_offset : low_offset + rank] w^T + bias)^(1/tau), in float32
   decayed_state_scan(proj, act_dtype, q_offset, k_offset, v_offset, q_scale, decay f32[T,heads*dk], states f32[slots,heads,dk,dv],
-                     slots i32[B], fresh bool[B]|None, q_start i32[B], q_len i32[B], heads, dk, dv) -> f32[T,heads*dv]
+                     slots i32[B], fresh bool[B]|None, q_start i32[B], q_len i32[B], heads, dk, dv) -> f32[S,T,heads*dv]
         per request and head, token by token: S = diag(decay_t) S + k_t v_t^T, o_t = S^T (q_t * q_scale); S is read from and
-        written to states[slots[b]] (fresh[b]: it starts at zero); q, k, v are columns of the product rows
+        written to states[slots[b]] (fresh[b]: it starts at zero); q, k, v are columns of the product rows; the output comes as
+        partial sums over ranges of the key channels (the backend's choice of S), which the consumer adds
   expert_mixture(x act[T,H], router act[E,H], router_bias act[E]|None, w_gate_up act[E,2F,H], w_down act[E,H,F], top) -> f32[T,H]
         float32 logits x router^T + bias, the `top` largest (lowest index among equals), softmax over those; the weighted
         sum of down_e(silu(gate_e x) * (up_e x)) over the chosen experts e, added in the order of the choices

@@ -28,7 +28,7 @@ def _load_library() -> ctypes.CDLL:
         lib = ctypes.CDLL(path)
     except (build.BuildError, OSError) as e:
         raise KernelsUnavailable(f"the HIP kernel library could not be built or loaded: {e}") from e
-    if lib.egpt_abi_version() != 20:
+    if lib.egpt_abi_version() != 21:
         raise KernelsUnavailable(f"{path} has an unexpected ABI version")
     return lib
 
@@ -113,7 +113,7 @@ class HipKernels(KernelBackend):
             "egpt_normed_pair_mean": [vp, i, vp, i, vp, vp, vp, vp, f, f, vp, i, i, i, vp],
             "egpt_tanh_cap": [vp, f, ctypes.c_longlong, vp],
             "egpt_whole_norm_store": [vp, i, i, vp, vp, vp, vp, f, vp, f, i, vp, vp, vp, i, i, i, i, i, i, i, vp],
-            "egpt_head_norm_gate": [vp, vp, f, vp, i, i, i, vp, i, i, i, i, vp],
+            "egpt_head_norm_gate": [vp, i, vp, f, vp, i, i, i, vp, i, i, i, i, vp],
             "egpt_channel_decay": [vp, i, i, i, i, vp, vp, f, vp, i, i, i, vp],
             "egpt_decayed_state_scan": [vp, i, i, i, i, i, f, vp, vp, vp, vp, vp, vp, i, i, vp, i, i, i, i, vp],
             "egpt_moe_route": [vp, vp, vp, vp, vp, i, i, i, i, i, vp],
@@ -122,6 +122,8 @@ class HipKernels(KernelBackend):
             "egpt_moe_down": [vp, vp, vp, vp, i, i, i, i, i, i, vp],
             "egpt_moe_combine": [vp, vp, vp, vp, i, i, i, vp],
         }
+        lib.egpt_scan_key_splits.restype = i
+        lib.egpt_scan_key_splits.argtypes = [i]
         lib.egpt_sample_workspace.restype = ctypes.c_size_t
         lib.egpt_sample_workspace.argtypes = [i, i]
         for name, argtypes in sigs.items():
@@ -1075,14 +1077,14 @@ class HipKernels(KernelBackend):
     def head_norm_gate(self, x, weight, eps, gate, gate_offset, out, heads, dv):
         t = out.shape[0]
         dt = self._act(out, "out")
-        self._need(x, "x", _F32, (t, heads * dv))
+        x_splits = self._product(x, "x", _F32, t, heads * dv)
         self._need(out, "out", None, (t, heads * dv))
         self._need(weight, "weight", out.dtype, (dv,))
         width = gate.shape[-1]
         splits = self._product(gate, "gate", out.dtype, t, width)
         if gate_offset < 0 or gate_offset + heads * dv > width:
             raise ValueError(f"gate columns {gate_offset}..{gate_offset + heads * dv} lie outside rows of {width} values")
-        self._run("egpt_head_norm_gate", x.data_ptr(), weight.data_ptr(), float(eps), gate.data_ptr(), splits, int(width),
+        self._run("egpt_head_norm_gate", x.data_ptr(), x_splits, weight.data_ptr(), float(eps), gate.data_ptr(), splits, int(width),
                   int(gate_offset), out.data_ptr(), t, heads, dv, dt, self._stream())
 
     # ------------------------------------------------------------------ a decaying matrix state per head
@@ -1120,9 +1122,7 @@ class HipKernels(KernelBackend):
         for off, n in ((q_offset, heads * dk), (k_offset, heads * dk), (v_offset, heads * dv)):
             if off < 0 or off + n > width:
                 raise ValueError(f"columns {off}..{off + n} lie outside rows of {width} values")
-        if dk > 256:
-            raise ValueError(f"key size {dk} is not supported by the state scan (at most 256)")
-        out = torch.empty((t, heads * dv), dtype=_F32, device=decay.device)
+        out = torch.empty((self.lib.egpt_scan_key_splits(dk), t, heads * dv), dtype=_F32, device=decay.device)
         self._run("egpt_decayed_state_scan", proj.data_ptr(), splits, int(width), int(q_offset), int(k_offset), int(v_offset),
                   float(q_scale), decay.data_ptr(), states.data_ptr(), slots.data_ptr(), self._ptr(fresh), q_start.data_ptr(),
                   q_len.data_ptr(), b, t, out.data_ptr(), heads, dk, dv, _DT[act_dtype], self._stream())

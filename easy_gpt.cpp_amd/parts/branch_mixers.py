@@ -143,8 +143,8 @@ class GatedLinearAttention(_Branch):
         tensors decide; this is what random weights draw).  names: tensor names behind `prefix`."""
         if not float(tau) > 0:
             raise ValueError(f"tau ({tau}) must be positive")
-        if not 0 < int(key_dim) <= 256:
-            raise ValueError(f"key size {key_dim} is not supported by the state scan (1 to 256)")
+        if not (0 < int(key_dim) <= 4096 and 0 < int(value_dim) <= 4096):
+            raise ValueError(f"key size {key_dim} / value size {value_dim} is not supported by the state scan (1 to 4096)")
         self.prefix, self.hidden_size = prefix, int(hidden_size)
         self.n_heads, self.key_dim, self.value_dim = int(n_heads), int(key_dim), int(value_dim)
         self.tau, self.eps, self.decay_rank = float(tau), float(eps), int(decay_rank)

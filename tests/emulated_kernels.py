@@ -251,7 +251,7 @@ class EmulatedKernels(KernelBackend):
 
     def head_norm_gate(self, x, weight, eps, gate, gate_offset, out, heads, dv):
         t = out.shape[0]
-        xx = x.to(F64).view(t, heads, dv)
+        xx = _whole(x).to(F64).view(t, heads, dv)
         xx = xx / torch.sqrt((xx * xx).mean(-1, keepdim=True) + eps) * weight.to(F64)
         g = _whole(gate)[:, gate_offset : gate_offset + heads * dv].to(F64)
         out.copy_((xx.reshape(t, heads * dv) * g * torch.sigmoid(g)).to(out.dtype))

@@ -41,6 +41,11 @@ def i32(*v):
     return torch.tensor(list(v), dtype=torch.int32, device=DEV)
 
 
+def added(o):
+    """What a scan leaves: partial sums [splits, T, W] over ranges of the key channels, added."""
+    return o.sum(0) if o.dim() == 3 else o
+
+
 # ----------------------------------------------------------------------------- stream operations
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_embedding_with_a_factor(k, dtype):
@@ -268,14 +273,14 @@ def test_a_batch_of_unequal_requests_gets_what_each_gets_alone(k):
 @pytest.mark.parametrize("heads, dv, splits", [(2, 24, 0), (3, 100, 2), (1, 64, 1)])
 def test_per_head_norm_with_the_silu_gate(k, dtype, heads, dv, splits):
     t, off, eps = 6, 5, 1e-5
-    x = rnd(t, heads * dv, seed=1, scale=3.0)
+    x = rnd(3, t, heads * dv, seed=1, scale=2.0) if splits == 2 else rnd(t, heads * dv, seed=1, scale=3.0)      # partial sums, or one tensor
     g = rnd(max(splits, 1), t, off + heads * dv + 3, seed=2)
     gate = g.sum(0) if splits else g[0].to(dtype).to(F64)
     w = (rnd(dv, seed=3) + 1).to(dtype)
     out = torch.empty((t, heads * dv), dtype=dtype, device=DEV)
     k.head_norm_gate(x.to(DEV), w.to(DEV), eps, g.to(DEV) if splits else g[0].to(dtype).to(DEV), off, out, heads, dv)
     gg = gate.to(F64)[:, off : off + heads * dv]
-    want = P.rms_norm(x.to(F64).view(t, heads, dv), w.to(F64), eps).reshape(t, -1) * gg * torch.sigmoid(gg)
+    want = P.rms_norm(added(x).to(F64).view(t, heads, dv), w.to(F64), eps).reshape(t, -1) * gg * torch.sigmoid(gg)
     close(out, want, dtype, "head norm and gate")
 
 
@@ -308,7 +313,7 @@ def plain_scan(whole, decay, offs, heads, dk, dv, q_scale, state=None):
 
 
 @pytest.mark.parametrize("heads, dk, dv", [(2, 6, 100), (3, 10, 12), (2, 16, 24), (1, 36, 70), (2, 64, 80), (4, 32, 48), (2, 128, 128),
-                                           (1, 160, 64), (1, 256, 16)])
+                                           (1, 160, 64), (1, 256, 16), (1, 300, 9)])
 def test_the_state_scan_whole_and_cut_anywhere(k, heads, dk, dv):
     t, q_scale = 150, dk ** -0.5
     proj, whole, decay, offs = scan_inputs(t, heads, dk, dv, 3, torch.float32, splits=2)
@@ -317,7 +322,7 @@ def test_the_state_scan_whole_and_cut_anywhere(k, heads, dk, dv):
     fresh = torch.tensor([True], device=DEV)
     got = k.decayed_state_scan(proj.to(DEV), torch.float32, *offs, q_scale, decay.to(DEV), states, i32(1), fresh, i32(0), i32(t),
                                heads, dk, dv)
-    close(got.view(t, heads, dv), want, torch.float32, "whole")
+    close(added(got).view(t, heads, dv), want, torch.float32, "whole")
     close(states[1], last, torch.float32, "the state it leaves")
     assert torch.isnan(states[0]).all() and torch.isnan(states[2]).all()
     # the same tokens in portions of changing size, down to single tokens: the same bits
@@ -329,7 +334,7 @@ def test_the_state_scan_whole_and_cut_anywhere(k, heads, dk, dv):
                                          torch.tensor([pos == 0], device=DEV), i32(0), i32(n), heads, dk, dv))
         pos += n
     assert pos == t
-    assert torch.equal(torch.cat(outs), got) and torch.equal(again[2], states[1])
+    assert torch.equal(torch.cat(outs, dim=-2), got) and torch.equal(again[2], states[1])
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
@@ -348,7 +353,7 @@ def test_the_state_scan_takes_a_rounded_product_and_a_batch_of_unequal_requests(
     for b, (s, n) in enumerate(zip(starts, lens)):
         start = None if bool(fresh[b]) else before[slots[b]].to(F64)
         want, last = plain_scan(rounded[s : s + n].to(F64), decay[s : s + n], offs, heads, dk, dv, q_scale, start)
-        close(got[s : s + n].view(n, heads, dv), want, torch.float32, f"request {b}")
+        close(added(got)[s : s + n].view(n, heads, dv), want, torch.float32, f"request {b}")
         close(states[slots[b]], last, torch.float32, f"state of request {b}")
     assert torch.equal(states[2].cpu(), before[2]) and torch.equal(states[5].cpu(), before[5])
 
@@ -371,9 +376,9 @@ def test_a_token_far_back_stays_in_a_state_that_does_not_decay(k):
                                          decay[first : first + n].to(DEV), states, i32(0), torch.tensor([first == 0], device=DEV),
                                          i32(0), i32(n), heads, dk, dv))
     want, _ = plain_scan(proj[0], decay, (0, dk, 2 * dk), heads, dk, dv, 1.0)
-    close(torch.cat(outs).view(t, heads, dv), want, torch.float32, "no decay")
+    close(torch.cat([added(o) for o in outs]).view(t, heads, dv), want, torch.float32, "no decay")
     found = 16.0 * proj[0, 17, 2 * dk :]
-    assert float((outs[-1][0].cpu() - found).abs().max()) < 0.01 * float(found.abs().max())
+    assert float((added(outs[-1])[0].cpu() - found).abs().max()) < 0.01 * float(found.abs().max())
 
 
 # ----------------------------------------------------------------------------- the mixture of experts
