@@ -79,6 +79,7 @@ struct ProductView {
     __device__ __forceinline__ bool present() const { return whole != nullptr || partial != nullptr; }
     __device__ __forceinline__ float at(size_t idx) const {
         if (n_splits == 0) return to_float(whole[idx]);
+        if (n_splits == 1) return partial[idx];          // a product written out in float32: one load, not a round of sixteen
         // up to sixteen loads in flight at a time (a chain of dependent kernels pays for round trips, not
         // bytes); the order of the additions is fixed
         float v = 0.f;
