@@ -1175,7 +1175,6 @@ class HipKernels(KernelBackend):
         self._run("egpt_moe_down", act.data_ptr(), w_down.data_ptr(), tiles.data_ptr(), y.data_ptr(), n_rows, hidden, ff,
                   experts, tile_rows, dt, st)
         self._run("egpt_moe_combine", y.data_ptr(), place.data_ptr(), weight.data_ptr(), out.data_ptr(), t, top, hidden, st)
-        self.last_routing = (chosen, weight)
         return out
 
     wide_rows_from = 16384          # rows of a step from which the window attention gives a wavefront 32 of them,

@@ -222,3 +222,47 @@ def test_the_residual_stream_after_every_layer(models, emulated):
     assert torch.equal(again, full)
     eng = Engine.from_dir(models["A"], dtype="float32", device="cpu", page_size=4, max_tokens=64, max_requests=1)
     H.assert_rows_match(H.replay(eng, H.trace_whole({"r0": tokens})), {"r0": full}, 1e-5, "streams")
+
+
+def test_each_branch_mixer_also_stands_alone_in_a_layer(emulated):
+    """A model described by hand: the attention with its distance bias alone in one layer (its output bias joins the
+    product there), the linear attention alone in the next; against the plain mechanisms."""
+    from easy_gpt.cpp_amd.parts import LayerSpec, ModelSpec, PartSpec, RunSpec
+
+    width, vocab, eps = 48, 50, 1e-5
+    norm = lambda prefix, name: PartSpec("layernorm", dict(eps=eps, name=name, bias_name=name + ".b"), prefix=prefix)
+    left = dict(heads=3, kv_heads=1, dim=8, vdim=12, scale=0.3, bias_max=7, q_temp=dict(coef=0.5, every=3))
+    right = dict(heads=2, dim=5, vdim=9, tau=2.0)
+    spec = ModelSpec(
+        hidden_size=width, vocab_size=vocab, max_position=1 << 20,
+        embedding=PartSpec("token_embedding_scaled", dict(scale=2.0, name="embed")),
+        layers=(
+            LayerSpec("pre_norm_mixer_only", PartSpec("distance_bias_attention", dict(
+                n_heads=3, n_kv_heads=1, key_dim=8, value_dim=12, scale=0.3, eps=eps, bias_far=7, bias_rows=6, query_growth=(0.5, 3)),
+                prefix="a."), None, {"mixer": norm("a.", "n")}),
+            LayerSpec("pre_norm_mixer_only", PartSpec("gated_linear_attention", dict(
+                n_heads=2, key_dim=5, value_dim=9, tau=2.0, eps=eps, decay_rank=3), prefix="b."), None, {"mixer": norm("b.", "n")}),
+        ),
+        run_order=(RunSpec(0, cache=0), RunSpec(1, state=0)),
+        final_norm=norm("", "fn"), output_head=PartSpec("linear_head", dict(tied=False, name="head")),
+    )
+    model = build_model(spec)
+    g = torch.Generator().manual_seed(3)
+    w = {}
+    for ps in model.param_specs():
+        t = torch.randn(ps.shape, generator=g) * (0.3 if len(ps.shape) > 1 else 0.5)
+        if ps.role == "norm_scale":
+            t = 1.0 + 0.2 * t
+        if ps.name == "b.a2.b":
+            t = t + 1.5
+        w[ps.name] = t.to(torch.bfloat16).to(torch.float32)
+    model.load(lambda name: w[name], torch.float32, "cpu")
+    eng = Engine(model, page_size=4, max_tokens=64, max_requests=2)
+    tokens = H.make_requests(vocab, [21], seed=4)["r0"]
+    w64 = {k: v.to(F64) for k, v in w.items()}
+    x = w64["embed"][torch.tensor(tokens)] * 2.0
+    x = x + P.biased_attention(P.layer_norm(x, w64["a.n"], w64["a.n.b"], eps), w64, "a.", left, eps)
+    x = x + P.gated_linear_attention(P.layer_norm(x, w64["b.n"], w64["b.n.b"], eps), w64, "b.", right, eps)
+    want = P.layer_norm(x, w64["fn"], w64["fn.b"], eps) @ w64["head"].T
+    for trace in (H.trace_whole({"r0": tokens}), H.trace_portions({"r0": tokens})):
+        H.assert_rows_match(H.replay(eng, trace), {"r0": want}, 1e-5, "branches alone")
