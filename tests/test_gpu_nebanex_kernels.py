@@ -107,7 +107,7 @@ def test_the_cap_on_logits(k):
 
 # ----------------------------------------------------------------------------- the left mixer's preparation
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("nq, nkv, dk, dv, splits, every", [(4, 2, 16, 32, 0, 4), (3, 3, 12, 20, 3, 1), (2, 1, 200, 8, 1, 0), (8, 1, 64, 48, 2, 96)])
+@pytest.mark.parametrize("nq, nkv, dk, dv, splits, every", [(4, 2, 16, 32, 0, 4), (3, 3, 12, 20, 3, 1), (2, 1, 200, 8, 1, 0), (8, 1, 64, 48, 2, 96), (40, 8, 96, 32, 1, 5)])
 def test_norms_over_the_whole_projection_the_query_factor_and_the_store(k, dtype, nq, nkv, dk, dv, splits, every):
     t, ps, eps, coef, extra = 13, 4, 1e-3, 0.4, 9
     used = (nq + nkv) * dk + nkv * dv
