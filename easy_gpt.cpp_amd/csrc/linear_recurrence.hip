@@ -100,7 +100,7 @@ __global__ __launch_bounds__(64 * kScanWaves) void decayed_state_scan_kernel(
             rq[u] = rk[u] = ra[u] = 0.f;
             if (tt < count && r < dk) {
                 const size_t row = static_cast<size_t>(t0 + base + tt);
-                rq[u] = proj.at(row * proj_width + q_off + h * dk + r) * q_scale;
+                rq[u] = proj.at(row * proj_width + q_off + h * dk + r);      // (scaled when it is staged: nothing here waits for a load)
                 rk[u] = proj.at(row * proj_width + k_off + h * dk + r);
                 ra[u] = decay[row * channels + h * dk + r];
             }
@@ -120,7 +120,7 @@ __global__ __launch_bounds__(64 * kScanWaves) void decayed_state_scan_kernel(
         __syncthreads();                          // the batch before is read, its parts are added
 #pragma unroll
         for (int u = 0; u < QKA; ++u) {
-            q_s[tid + u * THREADS] = rq[u];
+            q_s[tid + u * THREADS] = rq[u] * q_scale;
             k_s[tid + u * THREADS] = rk[u];
             a_s[tid + u * THREADS] = ra[u];
         }
